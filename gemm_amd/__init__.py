@@ -1,0 +1,102 @@
+"""gemm_amd — host-side mirror of the reference's extension surface over libneogemm.so.
+
+The drop-in module is `neoGEMM` (built by setup.py from csrc/neogemm_torch.cpp), with the reference's
+`neoGemmV1(A, B, C)` (nemgemmV03.cu:396-399) plus `C = gemm(A, B)`.  This package offers the same
+three functions through the C ABI with ctypes — which is what the parity tests and the bench use, so
+that every measured call crosses the plain-pointer boundary of include/neogemm.h — and lets tests
+force a kernel variant / split-K factor.
+
+Nothing here computes: without libneogemm.so and a GPU every call raises.
+"""
+import torch
+
+from . import _abi
+from ._abi import (B_KN, B_NK, C_COL, C_ROW, NeoGemmError, VARIANT_AUTO, VARIANT_GENERIC, VARIANT_NAMES,  # noqa: F401
+                   VARIANT_T128x128_W4, VARIANT_T128x256_W8, VARIANT_T256x128_W8, VARIANT_T256x256_W4,
+                   VARIANT_T256x256_W8, plan, strerror, version, workspace_bytes)
+
+__all__ = ["gemm", "neoGemmV1", "neogemm", "gemm_into", "plan", "workspace_bytes", "version", "NeoGemmError"]
+
+_workspaces = {}
+
+
+def _check(t, name):
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name} must be a torch.Tensor")
+    if not t.is_cuda:
+        raise ValueError(f"{name} must be a GPU tensor (there is no CPU path)")
+    if t.dtype != torch.bfloat16:
+        raise TypeError(f"{name} must be bfloat16, got {t.dtype}")
+    if t.dim() != 2:
+        raise ValueError(f"{name} must be 2-D, got {t.dim()}-D")
+
+
+def _workspace(device, nbytes):
+    ws = _workspaces.get(device)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+        _workspaces[device] = ws
+    return ws
+
+
+def gemm_into(A, B, C, M, N, K, lda, ldb, ldc, b_layout, c_layout, variant=None, split_k=0, group_m=0):
+    """Call the C ABI on torch's current stream; A, B, C are torch tensors used as device buffers."""
+    need = workspace_bytes(M, N, K)
+    if variant is not None and split_k > 1:
+        need = max(need, split_k * M * N * 4)
+    ws_ptr = 0
+    if need:
+        ws_ptr = _workspace(C.device, need).data_ptr()
+    with torch.cuda.device(C.device):
+        stream = torch.cuda.current_stream().cuda_stream
+        st = _abi.gemm_raw(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, lda, ldb, ldc, b_layout, c_layout,
+                           ws_ptr, need, stream, variant, split_k, group_m)
+    if st != _abi.OK:
+        raise NeoGemmError(st, f"M={M} N={N} K={K} b_layout={b_layout} c_layout={c_layout} variant={variant}")
+
+
+def gemm(A, B, variant=None, split_k=0, group_m=0):
+    """C[M,N] = A[M,K] @ B[K,N]; bf16 in, fp32 accumulate, bf16 out (new tensor)."""
+    _check(A, "A")
+    _check(B, "B")
+    if A.shape[1] != B.shape[0]:
+        raise ValueError(f"inner dimensions differ: A is {tuple(A.shape)}, B is {tuple(B.shape)}")
+    if A.device != B.device:
+        raise ValueError("A and B must be on the same device")
+    if A.stride(1) != 1 and A.shape[1] > 1:
+        A = A.contiguous()
+    M, K = A.shape
+    N = B.shape[1]
+    lda = A.stride(0) if M > 1 else max(K, 1)
+    if B.stride(1) == 1 or N <= 1:
+        b_layout, ldb = B_KN, (B.stride(0) if K > 1 else max(N, 1))
+    elif B.stride(0) == 1:
+        b_layout, ldb = B_NK, (B.stride(1) if N > 1 else max(K, 1))
+    else:
+        B = B.contiguous()
+        b_layout, ldb = B_KN, max(N, 1)
+    C = torch.empty((M, N), dtype=torch.bfloat16, device=A.device)
+    if M and N:
+        gemm_into(A, B, C, M, N, K, lda, ldb, max(N, 1), b_layout, C_ROW, variant, split_k, group_m)
+    return C
+
+
+def neoGemmV1(A, B, C, variant=None, split_k=0, group_m=0):
+    """Reference call (nemgemmV03.cu:343-391): A [M,K], B [N,K], C receives A @ B.T column-major."""
+    _check(A, "A")
+    _check(B, "B")
+    _check(C, "C")
+    if A.shape[1] != B.shape[1]:
+        raise ValueError(f"A is [M,K] and B is [N,K]: K differs ({A.shape[1]} vs {B.shape[1]})")
+    if not (A.is_contiguous() and B.is_contiguous() and C.is_contiguous()):
+        raise ValueError("A, B and C must be contiguous")
+    M, K = A.shape
+    N = B.shape[0]
+    if C.numel() != M * N:
+        raise ValueError(f"C must hold M*N = {M * N} elements, has {C.numel()}")
+    if M and N:
+        gemm_into(A, B, C, M, N, K, max(K, 1), max(K, 1), M, B_NK, C_COL, variant, split_k, group_m)
+    return None
+
+
+neogemm = neoGemmV1

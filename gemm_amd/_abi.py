@@ -1,0 +1,91 @@
+"""ctypes binding of the C ABI in include/neogemm.h (gemm_amd/libneogemm.so).
+
+This is the binding the parity tests call through: plain pointers and sizes, no torch types cross it.
+torch is used by callers only to own device memory and to name the stream.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libneogemm.so")
+
+OK, ERR_BAD_ARG, ERR_WORKSPACE, ERR_UNSUPPORTED, ERR_LAUNCH = 0, -1, -2, -3, -4
+B_KN, B_NK = 0, 1
+C_ROW, C_COL = 0, 1
+VARIANT_AUTO, VARIANT_GENERIC = 0, 1
+VARIANT_T256x256_W8, VARIANT_T256x256_W4, VARIANT_T128x128_W4 = 2, 3, 4
+VARIANT_T256x128_W8, VARIANT_T128x256_W8 = 5, 6
+VARIANT_COUNT = 7
+VARIANT_NAMES = {0: "auto", 1: "generic", 2: "256x256_w8", 3: "256x256_w4", 4: "128x128_w4", 5: "256x128_w8",
+                 6: "128x256_w8"}
+
+# every symbol include/neogemm.h declares, with its prototype
+_i64, _int, _vp, _sz = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t
+PROTOTYPES = {
+    "neogemm_bf16": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _vp, _sz, _vp]),
+    "neogemm_bf16_workspace_bytes": (_sz, [_i64, _i64, _i64]),
+    "neogemm_bf16_variant": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _vp, _sz, _vp,
+                                    _int, _int, _int]),
+    "neogemm_bf16_plan": (_int, [_i64, _i64, _i64, _int, _int, _int, ctypes.POINTER(_int), ctypes.POINTER(_int)]),
+    "neogemm_strerror": (ctypes.c_char_p, [_int]),
+    "neogemm_version": (ctypes.c_char_p, []),
+}
+
+_lib = None
+
+
+def load():
+    """Load libneogemm.so (built by `python setup.py build_ext --inplace` or __graft_entry__.build()).
+
+    There is no fallback: a missing library is an error, never a slower path.
+    """
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `python setup.py build_ext --inplace` "
+                "(hipcc --offload-arch=gfx950); there is no CPU or PyTorch fallback for the GEMM path")
+        lib = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in PROTOTYPES.items():
+            fn = getattr(lib, name)
+            fn.restype, fn.argtypes = res, args
+        _lib = lib
+    return _lib
+
+
+class NeoGemmError(RuntimeError):
+    def __init__(self, status, what=""):
+        self.status = status
+        msg = load().neogemm_strerror(status).decode()
+        super().__init__(f"neogemm status {status}: {msg}{(' (' + what + ')') if what else ''}")
+
+
+def strerror(status):
+    return load().neogemm_strerror(status).decode()
+
+
+def version():
+    return load().neogemm_version().decode()
+
+
+def workspace_bytes(M, N, K):
+    return int(load().neogemm_bf16_workspace_bytes(M, N, K))
+
+
+def plan(M, N, K, b_layout=B_KN, c_layout=C_ROW, aligned=True):
+    v, s = _int(0), _int(0)
+    st = load().neogemm_bf16_plan(M, N, K, b_layout, c_layout, int(aligned), ctypes.byref(v), ctypes.byref(s))
+    if st != OK:
+        raise NeoGemmError(st)
+    return v.value, s.value
+
+
+def gemm_raw(A_ptr, B_ptr, C_ptr, M, N, K, lda, ldb, ldc, b_layout, c_layout, ws_ptr=0, ws_bytes=0, stream=0,
+             variant=None, split_k=0, group_m=0):
+    """Thin call-through; returns the status code (no exception)."""
+    lib = load()
+    if variant is None:
+        return lib.neogemm_bf16(A_ptr, B_ptr, C_ptr, M, N, K, lda, ldb, ldc, b_layout, c_layout, ws_ptr or None,
+                                ws_bytes, stream or None)
+    return lib.neogemm_bf16_variant(A_ptr, B_ptr, C_ptr, M, N, K, lda, ldb, ldc, b_layout, c_layout,
+                                    ws_ptr or None, ws_bytes, stream or None, variant, split_k, group_m)

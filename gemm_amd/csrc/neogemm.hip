@@ -1,0 +1,641 @@
+// BF16 GEMM for MI355X (gfx950 / CDNA4): kernels and the C ABI declared in include/neogemm.h.
+//
+// What is computed is what the reference's kernel computes (v01.cu:189-270): every output element is
+// the fp32-accumulated dot product of a row of A with a row/column of B, rounded once to bf16 with
+// round-to-nearest-even.  How it is computed shares nothing with it: the reference stages 64x64 tiles
+// with TMA and issues WGMMA from one warpgroup (v01.cu:215-237); here a workgroup of wave64s owns a
+// 256x256 (or smaller) macro-tile, stages 64-deep K slabs with direct-to-LDS buffer loads into a
+// double-buffered, XOR-swizzled LDS image, and feeds v_mfma_f32_32x32x16_bf16 from ds_read_b128 /
+// ds_read_b64_tr_b16.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include <type_traits>
+
+#include "neogemm.h"
+
+namespace neogemm {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) int i32x4;
+typedef __attribute__((ext_vector_type(4))) short i16x4;
+typedef __attribute__((ext_vector_type(8))) short i16x8;
+
+#define NEOGEMM_AS3 __attribute__((address_space(3)))
+
+static constexpr int KT = 64;                      // K depth of one LDS stage (bf16 elements)
+static constexpr uint32_t OOB_OFFSET = 0x80000000u;  // >= every num_records this file builds
+
+// ---------------------------------------------------------------------------------------------
+// LDS image of an operand tile and its swizzles.
+//
+// K-major operand (rows of the matrix are K-contiguous: A[M,K], B[N,K]):
+//   image = ROWS x 128 B, row r at r*128, eight 16-byte chunks per row; logical chunk c of row r
+//   lives at physical chunk c ^ swz_k(r).  An MFMA operand read has 32 lanes fetch the same logical
+//   chunk of 32 consecutive rows; swz_k makes any 8 consecutive rows hit 8 distinct chunks and any
+//   16 consecutive rows hit 16 distinct 16-byte slots of a 256-byte window.
+// MN-major operand (the K index is the slow one: B[K,N]):
+//   image = 64 x (ROWS*2) B, k-row at k*ROWS*2; logical chunk c (8 columns) of k-row k lives at
+//   physical chunk c ^ swz_mn(k & 3).  Read back with ds_read_b64_tr_b16, whose 16-lane groups pull
+//   4 k-rows x 16 columns and hand lane j the 4 k-values of column j.
+// Direct-to-LDS loads write 64 lanes x 16 B contiguously, so the swizzle is applied by choosing which
+// global chunk each lane fetches.
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ uint32_t swz_k(uint32_t row) { return ((row >> 1) & 7u) ^ ((row & 1u) << 2); }
+__device__ __forceinline__ uint32_t swz_mn(uint32_t k4) {
+  // k4 in 0..3 -> {0, 4, 10, 14}
+  uint32_t u = (k4 << 1) ^ (k4 >> 1);
+  return u << 1;
+}
+
+// One 1 KiB direct-to-LDS load: lane i's 16 bytes at (rsrc.base + voff) land at lds + 16*i.
+// The compiler is not told that this touches LDS; ordering against ds_read is done by hand with
+// s_waitcnt vmcnt + s_barrier (a builtin load would make the compiler wait vmcnt(0) before every
+// LDS read and serialise the pipeline).
+__device__ __forceinline__ void dma16(i32x4 rsrc, uint32_t lds, uint32_t voff) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+               :
+               : "s"(lds), "v"(voff), "s"(rsrc)
+               : "memory");
+}
+
+__device__ __forceinline__ bf16x8 lds_read_b128(uint32_t addr) {
+  return *((NEOGEMM_AS3 bf16x8*)(uintptr_t)addr);
+}
+__device__ __forceinline__ i16x4 lds_read_tr16(uint32_t addr) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4i16((NEOGEMM_AS3 i16x4*)(uintptr_t)addr);
+}
+
+struct TileArgs {
+  const char* A;  // operand whose rows become output rows
+  const char* B;  // operand whose rows/columns become output columns
+  char* C;        // bf16 output, row-major [M][ldc]
+  float* ws;      // split-K partials [ksplit][M][N] fp32 (ksplit > 1 only)
+  int M, N, K;
+  long lda, ldb, ldc;  // elements
+  int ntm, ntn, group_m;
+  int ksplit, ktiles_per_split;
+};
+
+template <int ROWS, bool KMAJOR, int NW>
+struct Operand {
+  static constexpr int NINSTR = ROWS / 8;        // 1 KiB wave-loads per 64-deep tile
+  static constexpr int IPW = NINSTR / NW;        // per wave
+  static constexpr int ROWB = ROWS * 2;          // bytes per k-row of an MN-major image
+  static constexpr int CPR = ROWS / 8;           // 16-byte chunks per k-row (MN-major)
+  static constexpr int KR = 64 / CPR;            // k-rows per wave-load (MN-major)
+  static_assert(NINSTR % NW == 0, "tile loads must divide evenly over the waves");
+  static_assert(KMAJOR || ROWS >= 128, "MN-major swizzle needs >= 16 chunks per k-row");
+
+  uint32_t voff[IPW];
+  uint64_t base, end;
+  uint32_t kadv;
+  uint32_t lds_w;
+
+  __device__ __forceinline__ void init(const char* ptr, long ld, int rows_total, int r0, int k_begin, int K,
+                                       int wave, int lane) {
+    if constexpr (KMAJOR) {
+      base = (uint64_t)ptr + ((uint64_t)r0 * ld + k_begin) * 2;
+      end = (uint64_t)ptr + ((uint64_t)(rows_total - 1) * ld + K) * 2;
+      kadv = KT * 2;
+#pragma unroll
+      for (int j = 0; j < IPW; ++j) {
+        uint32_t row = (wave * IPW + j) * 8 + (lane >> 3);
+        uint32_t c = (lane & 7) ^ swz_k(row);
+        voff[j] = row * (uint32_t)ld * 2 + c * 16;
+      }
+    } else {
+      base = (uint64_t)ptr + ((uint64_t)k_begin * ld + r0) * 2;
+      end = (uint64_t)ptr + ((uint64_t)(K - 1) * ld + rows_total) * 2;
+      kadv = KT * (uint32_t)ld * 2;
+#pragma unroll
+      for (int j = 0; j < IPW; ++j) {
+        uint32_t krow = (wave * IPW + j) * KR + lane / CPR;
+        uint32_t c = (lane % CPR) ^ swz_mn(krow & 3);
+        voff[j] = krow * (uint32_t)ld * 2 + c * 16;
+        // A chunk that starts past the last column would wrap into the next k-row.
+        if (r0 + (int)c * 8 >= rows_total) voff[j] = OOB_OFFSET;
+      }
+    }
+    lds_w = wave * IPW * 1024;
+  }
+
+  // K-major only: drop the chunks of the last, partial K tile (they would wrap into the next row).
+  __device__ __forceinline__ void mask_k_tail(int krem, int wave, int lane) {
+    if constexpr (KMAJOR) {
+#pragma unroll
+      for (int j = 0; j < IPW; ++j) {
+        uint32_t row = (wave * IPW + j) * 8 + (lane >> 3);
+        uint32_t c = (lane & 7) ^ swz_k(row);
+        if ((int)c * 8 >= krem) voff[j] = OOB_OFFSET;
+      }
+    }
+  }
+
+  __device__ __forceinline__ void issue(uint32_t lds_tile) const {
+    const uint64_t rem = end - base;
+    const uint32_t nr = (rem >> 31) ? 0x80000000u : (uint32_t)rem;
+    i32x4 rsrc;
+    rsrc[0] = (int)(uint32_t)base;
+    rsrc[1] = (int)((uint32_t)(base >> 32) & 0xffffu);
+    rsrc[2] = (int)nr;
+    rsrc[3] = 0x00020000;
+#pragma unroll
+    for (int j = 0; j < IPW; ++j) dma16(rsrc, lds_tile + lds_w + j * 1024, voff[j]);
+  }
+  __device__ __forceinline__ void advance() { base += kadv; }
+};
+
+// Per-lane constants for reading MFMA operand fragments (32 rows x 16 k per fragment) out of the image.
+template <int ROWS, bool KMAJOR, int NT>
+struct FragReader {
+  static constexpr int ROWB = ROWS * 2;
+  uint32_t lane_off[KMAJOR ? 1 : NT];
+  uint32_t xs[KMAJOR ? 4 : 1];
+
+  __device__ __forceinline__ void init(int wrow0, int lane) {
+    if constexpr (KMAJOR) {
+      lane_off[0] = (uint32_t)(wrow0 + (lane & 31)) * 128;
+#pragma unroll
+      for (int s = 0; s < 4; ++s) xs[s] = (((uint32_t)(2 * s + (lane >> 5))) ^ swz_k(lane & 15)) << 4;
+    } else {
+      const uint32_t i = lane & 15, g1 = (lane >> 4) & 1, h = lane >> 5;
+      const uint32_t tr_r = i >> 2, tr_c = i & 3;
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        uint32_t chunk = (uint32_t)(wrow0 >> 3) + 4 * t + 2 * g1 + (tr_c >> 1);
+        lane_off[t] = (8 * h + tr_r) * ROWB + ((chunk ^ swz_mn(tr_r)) << 4) + ((tr_c & 1) << 3);
+      }
+      xs[0] = 0;
+    }
+  }
+  // fragment t (32 rows), k-step s (16 deep) of the tile image at LDS address `img`
+  __device__ __forceinline__ bf16x8 read(uint32_t img, int t, int s) const {
+    if constexpr (KMAJOR) {
+      return lds_read_b128(img + lane_off[0] + t * 4096 + xs[s]);
+    } else {
+      i16x4 lo = lds_read_tr16(img + lane_off[t] + (16 * s) * ROWB);
+      i16x4 hi = lds_read_tr16(img + lane_off[t] + (16 * s + 4) * ROWB);
+      i16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+      return __builtin_bit_cast(bf16x8, v);
+    }
+  }
+};
+
+template <int BM, int BN, int WGM, int WGN, bool AK, bool BK>
+__global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
+  constexpr int NW = WGM * WGN;
+  constexpr int WTM = BM / WGM, WTN = BN / WGN;
+  constexpr int TM = WTM / 32, TN = WTN / 32;
+  constexpr uint32_t A_BYTES = BM * 128, B_BYTES = BN * 128, STAGE = A_BYTES + B_BYTES;
+  static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be a multiple of the 32x32 MFMA tile");
+
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(NEOGEMM_AS3 char*)smem;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WGN, wn = wave % WGN;
+
+  // Workgroup id -> output tile.  Consecutive ids land on different XCDs (round-robin over the 8
+  // dies, each with its own L2), so id%8 selects a contiguous slice of the tile order, and the tile
+  // order itself walks group_m tile-rows at a time so a slice is a compact block of C.
+  int m0, n0;
+  {
+    const int total = p.ntm * p.ntn;
+    const int pid = blockIdx.x;
+    const int q = total >> 3, r = total & 7, x = pid & 7;
+    const int lin = x * q + (x < r ? x : r) + (pid >> 3);
+    const int per_group = p.group_m * p.ntn;
+    const int g = lin / per_group;
+    const int first = g * p.group_m;
+    const int gsz = (p.ntm - first) < p.group_m ? (p.ntm - first) : p.group_m;
+    const int rem = lin - g * per_group;
+    m0 = (first + rem % gsz) * BM;
+    n0 = (rem / gsz) * BN;
+  }
+  const int kz = blockIdx.y;
+  const int k_begin = kz * p.ktiles_per_split * KT;
+  int k_end = k_begin + p.ktiles_per_split * KT;
+  if (k_end > p.K) k_end = p.K;
+  const int nkt = (k_end - k_begin + KT - 1) / KT;
+  const int k_tail = (k_end - k_begin) - (nkt - 1) * KT;  // depth of the last tile, 1..64
+
+  Operand<BM, AK, NW> opa;
+  Operand<BN, BK, NW> opb;
+  opa.init(p.A, p.lda, p.M, m0, k_begin, p.K, wave, lane);
+  opb.init(p.B, p.ldb, p.N, n0, k_begin, p.K, wave, lane);
+  FragReader<BM, AK, TM> fa;
+  FragReader<BN, BK, TN> fb;
+  fa.init(wm * WTM, lane);
+  fb.init(wn * WTN, lane);
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  // tail_check: the tile being loaded may be the last, partial one (never true in the steady loop)
+  auto load_tile = [&](int kt, uint32_t stage, bool tail_check) {
+    if (tail_check && kt == nkt - 1 && k_tail != KT) {
+      opa.mask_k_tail(k_tail, wave, lane);
+      opb.mask_k_tail(k_tail, wave, lane);
+    }
+    opa.issue(lds0 + stage * STAGE);
+    opb.issue(lds0 + stage * STAGE + A_BYTES);
+    opa.advance();
+    opb.advance();
+  };
+
+  bf16x8 af[2][TM], bfr[2][TN];
+  auto read_frags = [&](int buf, uint32_t stage, int s) {
+    const uint32_t imgA = lds0 + stage * STAGE, imgB = imgA + A_BYTES;
+#pragma unroll
+    for (int t = 0; t < TM; ++t) af[buf][t] = fa.read(imgA, t, s);
+#pragma unroll
+    for (int t = 0; t < TN; ++t) bfr[buf][t] = fb.read(imgB, t, s);
+  };
+  auto mfma_step = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        // B fragment first: D rows index n, D columns index m, so a lane ends up with 4
+        // consecutive n of one output row (an 8-byte store) instead of 4 rows of one column.
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[buf][j], af[buf][i], acc[i][j], 0, 0, 0);
+  };
+  // LDS reads of the next k-step are issued two per MFMA at the head of the current step.
+  constexpr int NREAD = TM * (AK ? 1 : 2) + TN * (BK ? 1 : 2);
+  auto sched_step = [&]() {
+#pragma unroll
+    for (int i = 0; i < (NREAD + 1) / 2; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // 2 DS reads
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - (NREAD + 1) / 2, 0);
+  };
+
+  // One 64-deep K tile = 4 k-steps.  Fragments of step s+1 are fetched under the MFMAs of step s,
+  // across tile boundaries too: before the last step of a tile every wave waits for its own loads of
+  // the next tile and meets the others at the barrier; past it the next tile is readable everywhere
+  // and the current tile's image is dead (its last fragments are already in registers), so the tile
+  // after next is streamed into it while the last step's MFMAs run.
+  auto tile_body = [&](int kt, uint32_t stage, auto steady, bool has_next, bool has_next2) {
+    read_frags(1, stage, 1);
+    mfma_step(0);
+    sched_step();
+    read_frags(0, stage, 2);
+    mfma_step(1);
+    sched_step();
+    read_frags(1, stage, 3);
+    mfma_step(0);
+    sched_step();
+    if (decltype(steady)::value || has_next) {
+      __builtin_amdgcn_sched_barrier(0);  // keep step 2's MFMAs above the wait
+      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+      if (decltype(steady)::value || has_next2) load_tile(kt + 2, stage, !decltype(steady)::value);
+      __builtin_amdgcn_sched_barrier(0);
+      read_frags(0, stage ^ 1, 0);
+    }
+    mfma_step(1);
+    sched_step();
+  };
+
+  load_tile(0, 0, true);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+  if (nkt > 1) load_tile(1, 1, true);
+  read_frags(0, 0, 0);
+  int kt = 0;
+  for (; kt + 4 < nkt; kt += 2) {  // the tile loaded by the second body (kt + 3) is never the last
+    tile_body(kt, 0, std::true_type{}, true, true);
+    tile_body(kt + 1, 1, std::true_type{}, true, true);
+  }
+  for (; kt < nkt; ++kt) tile_body(kt, kt & 1, std::false_type{}, kt + 1 < nkt, kt + 2 < nkt);
+
+  // Epilogue: lane holds, per 32x32 tile, output row (lane & 31) and four runs of 4 consecutive columns.
+  const int row_l = lane & 31, colq = (lane >> 5) * 4;
+  if (p.ksplit == 1) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int row = m0 + wm * WTM + i * 32 + row_l;
+      if (row >= p.M) continue;
+      char* crow = p.C + (size_t)row * p.ldc * 2;
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+          const int col = n0 + wn * WTN + j * 32 + 8 * b + colq;
+          bf16x4 o;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) o[r] = (__bf16)acc[i][j][4 * b + r];
+          if (col + 3 < p.N) {
+            *(bf16x4*)(crow + (size_t)col * 2) = o;
+          } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+              if (col + r < p.N) *(__bf16*)(crow + (size_t)(col + r) * 2) = o[r];
+          }
+        }
+      }
+    }
+  } else {
+    float* wsz = p.ws + (size_t)kz * p.M * p.N;
+    const bool vec = (p.N & 3) == 0;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int row = m0 + wm * WTM + i * 32 + row_l;
+      if (row >= p.M) continue;
+      float* wrow = wsz + (size_t)row * p.N;
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+          const int col = n0 + wn * WTN + j * 32 + 8 * b + colq;
+          if (vec && col + 3 < p.N) {
+            f32x4 o = {acc[i][j][4 * b], acc[i][j][4 * b + 1], acc[i][j][4 * b + 2], acc[i][j][4 * b + 3]};
+            *(f32x4*)(wrow + col) = o;
+          } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+              if (col + r < p.N) wrow[col + r] = acc[i][j][4 * b + r];
+          }
+        }
+      }
+    }
+  }
+}
+
+// Sum the split-K partials in split order (deterministic) and round once to bf16.
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ ws, char* C, int M, int N,
+                                                            long ldc, int ksplit) {
+  const size_t MN = (size_t)M * N;
+  const size_t idx = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
+  if (idx >= MN) return;
+  if ((N & 3) == 0) {
+    f32x4 s = *(const f32x4*)(ws + idx);
+    for (int z = 1; z < ksplit; ++z) {
+      f32x4 t = *(const f32x4*)(ws + z * MN + idx);
+      s[0] += t[0];
+      s[1] += t[1];
+      s[2] += t[2];
+      s[3] += t[3];
+    }
+    const size_t row = idx / N, col = idx - row * N;
+    bf16x4 o = {(__bf16)s[0], (__bf16)s[1], (__bf16)s[2], (__bf16)s[3]};
+    *(bf16x4*)(C + (row * ldc + col) * 2) = o;
+  } else {
+    for (int e = 0; e < 4 && idx + e < MN; ++e) {
+      float s = ws[idx + e];
+      for (int z = 1; z < ksplit; ++z) s += ws[z * MN + idx + e];
+      const size_t row = (idx + e) / N, col = (idx + e) - row * N;
+      *(__bf16*)(C + (row * ldc + col) * 2) = (__bf16)s;
+    }
+  }
+}
+
+// Fallback for anything the tile kernels do not take: arbitrary element strides, no alignment needs.
+// One thread per output element, 16x16 outputs per workgroup, K walked 16 at a time through LDS.
+__global__ __launch_bounds__(256) void gemm_generic_kernel(const __bf16* __restrict__ A, const __bf16* __restrict__ B,
+                                                           __bf16* C, int M, int N, int K, long sam, long sak,
+                                                           long sbk, long sbn, long scm, long scn) {
+  __shared__ float sa[16][17];
+  __shared__ float sb[16][17];
+  const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+  const long row = (long)blockIdx.y * 16 + ty, col = (long)blockIdx.x * 16 + tx;
+  float acc = 0.f;
+  for (int k0 = 0; k0 < K; k0 += 16) {
+    // sa[ty][tx] = A(row, k0+tx); sb[ty][tx] = B(k0+ty, col)
+    sa[ty][tx] = (row < M && k0 + tx < K) ? (float)A[row * sam + (long)(k0 + tx) * sak] : 0.f;
+    sb[ty][tx] = (col < N && k0 + ty < K) ? (float)B[(long)(k0 + ty) * sbk + col * sbn] : 0.f;
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < 16; ++k) acc = __builtin_fmaf(sa[ty][k], sb[k][tx], acc);
+    __syncthreads();
+  }
+  if (row < M && col < N) C[row * scm + col * scn] = (__bf16)acc;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Host side
+// ---------------------------------------------------------------------------------------------
+struct VariantInfo {
+  int bm, bn, nwaves;
+};
+static const VariantInfo kVariants[NEOGEMM_VARIANT_COUNT] = {
+    {0, 0, 0}, {16, 16, 4}, {256, 256, 8}, {256, 256, 4}, {128, 128, 4}, {256, 128, 8}, {128, 256, 8},
+};
+
+template <int BM, int BN, int WGM, int WGN>
+static hipError_t launch_tile(const TileArgs& a, bool ak, bool bk, hipStream_t st) {
+  constexpr size_t lds = 2 * (size_t)(BM + BN) * 128;
+  dim3 grid(a.ntm * a.ntn, a.ksplit), block(WGM * WGN * 64);
+  auto go = [&](auto kern) -> hipError_t {
+    static bool attr_done = false;  // per instantiation
+    if (!attr_done) {
+      hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      if (e != hipSuccess) return e;
+      attr_done = true;
+    }
+    kern<<<grid, block, lds, st>>>(a);
+    return hipGetLastError();
+  };
+  if (ak && bk) return go(gemm_tile_kernel<BM, BN, WGM, WGN, true, true>);
+  if (ak && !bk) {
+    if constexpr (BN >= 128) return go(gemm_tile_kernel<BM, BN, WGM, WGN, true, false>);
+  }
+  if (!ak && bk) {
+    if constexpr (BM >= 128) return go(gemm_tile_kernel<BM, BN, WGM, WGN, false, true>);
+  }
+  return hipErrorInvalidValue;
+}
+
+static bool is_aligned(const void* A, const void* B, const void* C, int64_t K, int64_t lda, int64_t ldb,
+                       int64_t ldc) {
+  return (((uintptr_t)A | (uintptr_t)B) & 15) == 0 && ((uintptr_t)C & 7) == 0 && (K & 7) == 0 && (lda & 7) == 0 &&
+         (ldb & 7) == 0 && (ldc & 3) == 0;
+}
+
+static int ceil_div(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
+
+// Shape -> (variant, split_k).  256 CUs; a 256x256 workgroup fills one CU (128 KiB of LDS).
+static void plan(int64_t M, int64_t N, int64_t K, bool aligned, int* variant, int* split_k) {
+  if (!aligned || K == 0) {
+    *variant = NEOGEMM_VARIANT_GENERIC;
+    *split_k = 1;
+    return;
+  }
+  int v = NEOGEMM_VARIANT_T256x256_W8;
+  if (M <= 128 || N <= 128 || (int64_t)ceil_div(M, 256) * ceil_div(N, 256) < 64) v = NEOGEMM_VARIANT_T128x128_W4;
+  const int64_t tiles = (int64_t)ceil_div(M, kVariants[v].bm) * ceil_div(N, kVariants[v].bn);
+  const int64_t ktiles = ceil_div(K, KT);
+  int s = 1;
+  if (tiles < 192) {
+    // not enough tiles to fill the chip: split K until there are ~2 workgroups per CU, keeping >= 4
+    // K tiles per split so the pipeline has something to overlap
+    int64_t want = (512 + tiles - 1) / tiles;
+    int64_t maxs = ktiles / 4 > 0 ? ktiles / 4 : 1;
+    s = (int)(want < maxs ? want : maxs);
+    if (s < 1) s = 1;
+    if (s > 64) s = 64;
+  }
+  *variant = v;
+  *split_k = s;
+}
+
+static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
+               int64_t ldc, int b_layout, int c_layout, void* workspace, size_t workspace_bytes, void* hip_stream,
+               int variant, int split_k, int group_m) {
+  if (M < 0 || N < 0 || K < 0) return NEOGEMM_ERR_BAD_ARG;
+  if ((b_layout != NEOGEMM_B_KN && b_layout != NEOGEMM_B_NK) || (c_layout != NEOGEMM_C_ROW && c_layout != NEOGEMM_C_COL))
+    return NEOGEMM_ERR_BAD_ARG;
+  if (variant < 0 || variant >= NEOGEMM_VARIANT_COUNT || split_k < 0 || group_m < 0) return NEOGEMM_ERR_BAD_ARG;
+  if (M == 0 || N == 0) return NEOGEMM_OK;
+  if (!C || (K > 0 && (!A || !B))) return NEOGEMM_ERR_BAD_ARG;
+  if (lda < K || ldb < (b_layout == NEOGEMM_B_KN ? N : K) || ldc < (c_layout == NEOGEMM_C_ROW ? N : M))
+    return NEOGEMM_ERR_BAD_ARG;
+  if (M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff) return NEOGEMM_ERR_BAD_ARG;
+  hipStream_t st = (hipStream_t)hip_stream;
+
+  // ld limits keep every in-tile byte offset below 2^31 (the buffer range check uses 32-bit offsets)
+  const bool aligned = is_aligned(A, B, C, K, lda, ldb, ldc) && lda < (1 << 21) && ldb < (1 << 21) && K > 0;
+  int v = variant, s = split_k;
+  if (v == NEOGEMM_VARIANT_AUTO) {
+    int pv, ps;
+    plan(M, N, K, aligned, &pv, &ps);
+    v = pv;
+    if (s == 0) s = ps;
+  }
+  if (s == 0) s = 1;
+
+  if (v == NEOGEMM_VARIANT_GENERIC) {
+    const long sbk = b_layout == NEOGEMM_B_KN ? ldb : 1, sbn = b_layout == NEOGEMM_B_KN ? 1 : ldb;
+    const long scm = c_layout == NEOGEMM_C_ROW ? ldc : 1, scn = c_layout == NEOGEMM_C_ROW ? 1 : ldc;
+    dim3 grid(ceil_div(N, 16), ceil_div(M, 16));
+    if (grid.y > 65535u * 16u) return NEOGEMM_ERR_UNSUPPORTED;
+    gemm_generic_kernel<<<grid, 256, 0, st>>>((const __bf16*)A, (const __bf16*)B, (__bf16*)C, (int)M, (int)N, (int)K,
+                                              lda, 1, sbk, sbn, scm, scn);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+      fprintf(stderr, "neogemm: generic kernel launch failed: %s\n", hipGetErrorString(e));
+      return NEOGEMM_ERR_LAUNCH;
+    }
+    return NEOGEMM_OK;
+  }
+
+  if (!aligned) return NEOGEMM_ERR_UNSUPPORTED;
+
+  // The tile kernels write row-major output.  Column-major C is the row-major transpose, i.e. the
+  // product with the operands' roles exchanged.
+  TileArgs a;
+  bool ak, bk;
+  if (c_layout == NEOGEMM_C_ROW) {
+    a.A = (const char*)A; a.lda = lda; ak = true; a.M = (int)M;
+    a.B = (const char*)B; a.ldb = ldb; bk = (b_layout == NEOGEMM_B_NK); a.N = (int)N;
+  } else {
+    a.A = (const char*)B; a.lda = ldb; ak = (b_layout == NEOGEMM_B_NK); a.M = (int)N;
+    a.B = (const char*)A; a.ldb = lda; bk = true; a.N = (int)M;
+  }
+  a.C = (char*)C;
+  a.ldc = ldc;
+  a.K = (int)K;
+  const VariantInfo& vi = kVariants[v];
+  if ((!ak && vi.bm < 128) || (!bk && vi.bn < 128)) return NEOGEMM_ERR_UNSUPPORTED;
+  a.ntm = ceil_div(a.M, vi.bm);
+  a.ntn = ceil_div(a.N, vi.bn);
+  if ((int64_t)a.ntm * a.ntn > 0x7fffffff) return NEOGEMM_ERR_UNSUPPORTED;
+  a.group_m = group_m > 0 ? group_m : 8;
+  const int ktiles = ceil_div(K, KT);
+  if (s > ktiles) s = ktiles;
+  a.ktiles_per_split = ceil_div(ktiles, s);
+  a.ksplit = ceil_div(ktiles, a.ktiles_per_split);  // no empty split
+  a.ws = nullptr;
+  if (a.ksplit > 1) {
+    const size_t need = (size_t)a.ksplit * (size_t)M * (size_t)N * sizeof(float);
+    if (!workspace || workspace_bytes < need) return NEOGEMM_ERR_WORKSPACE;
+    if (((uintptr_t)workspace & 15) != 0) return NEOGEMM_ERR_BAD_ARG;
+    a.ws = (float*)workspace;
+  }
+
+  hipError_t e;
+  switch (v) {
+    case NEOGEMM_VARIANT_T256x256_W8: e = launch_tile<256, 256, 2, 4>(a, ak, bk, st); break;
+    case NEOGEMM_VARIANT_T256x256_W4: e = launch_tile<256, 256, 2, 2>(a, ak, bk, st); break;
+    case NEOGEMM_VARIANT_T128x128_W4: e = launch_tile<128, 128, 2, 2>(a, ak, bk, st); break;
+    case NEOGEMM_VARIANT_T256x128_W8: e = launch_tile<256, 128, 4, 2>(a, ak, bk, st); break;
+    case NEOGEMM_VARIANT_T128x256_W8: e = launch_tile<128, 256, 2, 4>(a, ak, bk, st); break;
+    default: return NEOGEMM_ERR_BAD_ARG;
+  }
+  if (e != hipSuccess) {
+    fprintf(stderr, "neogemm: tile kernel launch failed (variant %d): %s\n", v, hipGetErrorString(e));
+    return NEOGEMM_ERR_LAUNCH;
+  }
+  if (a.ksplit > 1) {
+    const size_t MN = (size_t)a.M * a.N;
+    const unsigned blocks = (unsigned)((MN + 1023) / 1024);
+    splitk_reduce_kernel<<<blocks, 256, 0, st>>>(a.ws, a.C, a.M, a.N, a.ldc, a.ksplit);
+    e = hipGetLastError();
+    if (e != hipSuccess) {
+      fprintf(stderr, "neogemm: split-K reduce launch failed: %s\n", hipGetErrorString(e));
+      return NEOGEMM_ERR_LAUNCH;
+    }
+  }
+  return NEOGEMM_OK;
+}
+
+}  // namespace neogemm
+
+extern "C" {
+
+int neogemm_bf16(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
+                 int64_t ldc, int b_layout, int c_layout, void* workspace, size_t workspace_bytes, void* hip_stream) {
+  return neogemm::run(A, B, C, M, N, K, lda, ldb, ldc, b_layout, c_layout, workspace, workspace_bytes, hip_stream,
+                      NEOGEMM_VARIANT_AUTO, 0, 0);
+}
+
+int neogemm_bf16_variant(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int64_t lda,
+                         int64_t ldb, int64_t ldc, int b_layout, int c_layout, void* workspace,
+                         size_t workspace_bytes, void* hip_stream, int variant, int split_k, int group_m) {
+  return neogemm::run(A, B, C, M, N, K, lda, ldb, ldc, b_layout, c_layout, workspace, workspace_bytes, hip_stream,
+                      variant, split_k, group_m);
+}
+
+size_t neogemm_bf16_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  if (M <= 0 || N <= 0 || K <= 0) return 0;
+  int v, s;
+  neogemm::plan(M, N, K, true, &v, &s);
+  return s > 1 ? (size_t)s * (size_t)M * (size_t)N * sizeof(float) : 0;
+}
+
+int neogemm_bf16_plan(int64_t M, int64_t N, int64_t K, int b_layout, int c_layout, int aligned, int* variant,
+                      int* split_k) {
+  (void)b_layout;
+  (void)c_layout;
+  if (!variant || !split_k || M < 0 || N < 0 || K < 0) return NEOGEMM_ERR_BAD_ARG;
+  neogemm::plan(M, N, K, aligned != 0, variant, split_k);
+  return NEOGEMM_OK;
+}
+
+const char* neogemm_strerror(int status) {
+  switch (status) {
+    case NEOGEMM_OK: return "success";
+    case NEOGEMM_ERR_BAD_ARG: return "bad argument (null pointer, negative size, leading dimension too small or unknown layout)";
+    case NEOGEMM_ERR_WORKSPACE: return "workspace missing or too small (see neogemm_bf16_workspace_bytes)";
+    case NEOGEMM_ERR_UNSUPPORTED: return "the requested kernel variant cannot run this shape or alignment";
+    case NEOGEMM_ERR_LAUNCH: return "HIP kernel launch failed";
+    default: return "unknown neogemm status";
+  }
+}
+
+const char* neogemm_version(void) { return "neogemm 0.1 gfx950"; }
+
+}  // extern "C"

@@ -1,0 +1,114 @@
+// Python module `neoGEMM`: the PyTorch-ROCm face of libneogemm.so.
+//
+// Keeps the reference's extension surface — module neoGEMM, function neoGemmV1(A, B, C) with keyword
+// names A, B, C returning None (nemgemmV03.cu:343-399, neogemmv4.cu:335-338), the older
+// neogemm(A, B, C) (v01.cu:272-317, neogemmV02.cu:304-307) — and adds C = gemm(A, B).  This file
+// only unwraps tensors, checks them and calls the C ABI of include/neogemm.h on torch's current HIP
+// stream; there is no kernel code and no HIP call here apart from asking torch for that stream.
+//
+// Differences from the reference launcher, on purpose:
+//  * arguments are validated (the reference only checks dtype through data_ptr<>, nemgemmV03.cu:349-351)
+//    and failures raise instead of printing to stderr (nemgemmV03.cu:387-390);
+//  * the launch goes to torch's current stream, not the legacy default stream (nemgemmV03.cu:383);
+//  * no state is cached between calls (the reference caches TMA descriptors keyed on shape only,
+//    nemgemmV03.cu:27-30,359-371, which goes stale when another tensor of the same shape is passed).
+#include <c10/hip/HIPGuard.h>
+#include <c10/hip/HIPStream.h>
+#include <torch/extension.h>
+
+#include <string>
+#include <vector>
+
+#include "neogemm.h"
+
+namespace {
+
+void check_operand(const torch::Tensor& t, const char* name) {
+  TORCH_CHECK(t.defined(), name, " is undefined");
+  TORCH_CHECK(t.is_cuda(), name, " must be a GPU tensor");
+  TORCH_CHECK(t.scalar_type() == at::kBFloat16, name, " must be bfloat16, got ", t.scalar_type());
+  TORCH_CHECK(t.dim() == 2, name, " must be 2-D, got ", t.dim(), "-D");
+}
+
+// A 2-D tensor whose rows are contiguous (stride(1) == 1) is passed with ld = stride(0).
+bool row_major(const torch::Tensor& t) { return t.size(1) <= 1 || t.stride(1) == 1; }
+int64_t row_ld(const torch::Tensor& t) { return t.size(0) <= 1 ? std::max<int64_t>(t.size(1), 1) : t.stride(0); }
+
+// Per-device split-K scratch.  Grown on demand through torch's caching allocator and kept; launches
+// on one stream are ordered, and a tensor replaced here stays alive until the stream that used it has
+// passed (the caching allocator defers reuse of blocks recorded on a stream).
+torch::Tensor& workspace_for(const torch::Tensor& like, size_t bytes) {
+  static thread_local std::vector<torch::Tensor> ws(64);
+  const int dev = like.get_device();
+  TORCH_CHECK(dev >= 0 && dev < 64, "unexpected device index ", dev);
+  if (!ws[dev].defined() || (size_t)ws[dev].numel() < bytes) {
+    ws[dev] = torch::empty({(int64_t)bytes}, like.options().dtype(torch::kUInt8));
+  }
+  return ws[dev];
+}
+
+void run(const torch::Tensor& A, const torch::Tensor& B, torch::Tensor& C, int64_t M, int64_t N, int64_t K,
+         int64_t lda, int64_t ldb, int64_t ldc, int b_layout, int c_layout) {
+  c10::hip::HIPGuard guard(A.device());
+  const size_t need = neogemm_bf16_workspace_bytes(M, N, K);
+  void* ws = nullptr;
+  if (need) ws = workspace_for(A, need).data_ptr();
+  hipStream_t stream = c10::hip::getCurrentHIPStream(A.get_device()).stream();
+  const int st = neogemm_bf16(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, lda, ldb, ldc, b_layout, c_layout,
+                              ws, need, (void*)stream);
+  TORCH_CHECK(st == NEOGEMM_OK, "neogemm_bf16 failed: ", neogemm_strerror(st));
+}
+
+// C = gemm(A, B): A [M,K], B [K,N] -> new C [M,N], all bf16.  A transposed view of a contiguous
+// [N,K] tensor is taken as is (that is the reference's own B layout), anything else is made contiguous.
+torch::Tensor gemm(torch::Tensor A, torch::Tensor B) {
+  check_operand(A, "A");
+  check_operand(B, "B");
+  TORCH_CHECK(A.device() == B.device(), "A and B must be on the same device");
+  TORCH_CHECK(A.size(1) == B.size(0), "inner dimensions differ: A is ", A.sizes(), ", B is ", B.sizes());
+  if (!row_major(A)) A = A.contiguous();
+  int b_layout = NEOGEMM_B_KN;
+  int64_t ldb;
+  if (row_major(B)) {
+    ldb = row_ld(B);
+  } else if (B.stride(0) == 1) {  // B = W.t() with W [N,K] row-major
+    b_layout = NEOGEMM_B_NK;
+    ldb = B.size(1) <= 1 ? std::max<int64_t>(B.size(0), 1) : B.stride(1);
+  } else {
+    B = B.contiguous();
+    ldb = row_ld(B);
+  }
+  const int64_t M = A.size(0), K = A.size(1), N = B.size(1);
+  torch::Tensor C = torch::empty({M, N}, A.options());
+  if (M == 0 || N == 0) return C;
+  run(A, B, C, M, N, K, row_ld(A), ldb, std::max<int64_t>(N, 1), b_layout, NEOGEMM_C_ROW);
+  return C;
+}
+
+// neoGemmV1(A, B, C): A [M,K], B [N,K], C holds M*N bf16 and receives the product column-major,
+// so that C.t() (viewing the [M,N]-shaped C of benchmark.py:12 transposed, benchmark.py:25) equals
+// A @ B.t() (benchmark.py:18) when M == N, and C.view(N, M).t() does in general.
+void neoGemmV1(torch::Tensor A, torch::Tensor B, torch::Tensor C) {
+  check_operand(A, "A");
+  check_operand(B, "B");
+  check_operand(C, "C");
+  TORCH_CHECK(A.device() == B.device() && A.device() == C.device(), "A, B and C must be on the same device");
+  TORCH_CHECK(A.size(1) == B.size(1), "A is [M,K] and B is [N,K]: K differs (", A.size(1), " vs ", B.size(1), ")");
+  TORCH_CHECK(A.is_contiguous() && B.is_contiguous() && C.is_contiguous(), "A, B and C must be contiguous");
+  const int64_t M = A.size(0), K = A.size(1), N = B.size(0);
+  TORCH_CHECK(C.numel() == M * N, "C must hold M*N = ", M * N, " elements, has ", C.numel());
+  if (M == 0 || N == 0) return;
+  run(A, B, C, M, N, K, std::max<int64_t>(K, 1), std::max<int64_t>(K, 1), M, NEOGEMM_B_NK, NEOGEMM_C_COL);
+}
+
+}  // namespace
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+  m.doc() = "BF16 GEMM for MI355X (gfx950): bf16 in, fp32 accumulate, bf16 out";
+  m.def("gemm", &gemm, "C[M,N] = A[M,K] @ B[K,N]", py::arg("A"), py::arg("B"));
+  m.def("neoGemmV1", &neoGemmV1, "C (column-major) = A[M,K] @ B[N,K]^T, in place", py::arg("A"), py::arg("B"),
+        py::arg("C"));
+  m.def("neogemm", &neoGemmV1, "alias of neoGemmV1 (the reference's first module name)", py::arg("A"),
+        py::arg("B"), py::arg("C"));
+  m.def("version", []() { return std::string(neogemm_version()); });
+}

@@ -1,0 +1,107 @@
+/*
+ * neogemm.h — C ABI of the MI355X (gfx950) BF16 GEMM library `libneogemm.so`.
+ *
+ * This is the boundary a replacement for the reference's extension binds to.
+ * The reference has no C layer of its own: its pybind11 functions take
+ * torch::Tensor directly (nemgemmV03.cu:343-399, v01.cu:272-317).  Every entry
+ * point below therefore cites the reference interface whose work it carries out.
+ *
+ * All pointers are DEVICE pointers unless stated otherwise; all matrices are
+ * bf16 (IEEE bfloat16, 2 bytes).  The product is accumulated in fp32 and
+ * rounded once to bf16 with round-to-nearest-even, as the reference's epilogue
+ * does (v01.cu:254-262, __float2bfloat16).
+ *
+ * Calls are asynchronous on `hip_stream` (a hipStream_t passed as void*; NULL
+ * is the default stream).  No entry point synchronises the host.
+ */
+#ifndef NEOGEMM_H
+#define NEOGEMM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Status codes (0 = success, negative = failure; never a HIP error enum). */
+#define NEOGEMM_OK 0
+#define NEOGEMM_ERR_BAD_ARG (-1)      /* null pointer, negative size, ld too small, unknown layout */
+#define NEOGEMM_ERR_WORKSPACE (-2)    /* workspace missing or smaller than neogemm_bf16_workspace_bytes */
+#define NEOGEMM_ERR_UNSUPPORTED (-3)  /* the forced variant cannot run this shape / alignment */
+#define NEOGEMM_ERR_LAUNCH (-4)       /* HIP refused the launch (see stderr for hipGetErrorString) */
+
+/* b_layout values */
+#define NEOGEMM_B_KN 0 /* B is [K,N] row-major (N contiguous): the layout `C = gemm(A, B)` is quoted on */
+#define NEOGEMM_B_NK 1 /* B is [N,K] row-major (K contiguous): the reference's layout, N = B.size(0)
+                          (nemgemmV03.cu:346), C = A * B^T (v01.cu:232-235) */
+/* c_layout values */
+#define NEOGEMM_C_ROW 0 /* C(i,j) at C[i*ldc + j] */
+#define NEOGEMM_C_COL 1 /* C(i,j) at C[j*ldc + i]: what the reference's epilogue writes (v01.cu:246,252) */
+
+/* Kernel variants for neogemm_bf16_variant(); 0 lets the library choose. */
+#define NEOGEMM_VARIANT_AUTO 0
+#define NEOGEMM_VARIANT_GENERIC 1   /* scalar-load fallback: any shape, stride, alignment */
+#define NEOGEMM_VARIANT_T256x256_W8 2 /* 256x256x64 macro-tile, 8 wave64 (2x4), 32x32x16 MFMA */
+#define NEOGEMM_VARIANT_T256x256_W4 3 /* 256x256x64 macro-tile, 4 wave64 (2x2) */
+#define NEOGEMM_VARIANT_T128x128_W4 4 /* 128x128x64 macro-tile, 4 wave64 (2x2) */
+#define NEOGEMM_VARIANT_T256x128_W8 5 /* 256x128x64 macro-tile, 8 wave64 (4x2) */
+#define NEOGEMM_VARIANT_T128x256_W8 6 /* 128x256x64 macro-tile, 8 wave64 (2x4) */
+#define NEOGEMM_VARIANT_COUNT 7
+
+/*
+ * C = A * op(B), bf16 in, fp32 accumulate, bf16 out.
+ * Replaces the host launcher neoGemmV1(A,B,C) (nemgemmV03.cu:343-391; v1/v2: neogemm(),
+ * v01.cu:272-313) together with the kernel it launches (v01.cu:189-270).  The reference call is
+ * neogemm_bf16(A,B,C, M,N,K, K,K,M, NEOGEMM_B_NK, NEOGEMM_C_COL, ws, ws_bytes, stream).
+ *
+ *   A          [M,K] row-major, leading dimension lda >= K (elements)
+ *   B          [K,N] with ldb >= N (b_layout 0) or [N,K] with ldb >= K (b_layout 1)
+ *   C          [M,N] row-major with ldc >= N (c_layout 0) or column-major with ldc >= M (c_layout 1)
+ *   workspace  device scratch of at least neogemm_bf16_workspace_bytes(M,N,K) bytes, or NULL when
+ *              that function returns 0 for the shape.  Only split-K paths use it (fp32 partials).
+ *
+ * Unlike the reference (M,N,K % 64 == 0, nemgemmV03.cu:375) every M,N,K >= 0 is accepted; shapes or
+ * pointers that the MFMA path cannot take (K % 8, ld % 8, 16-byte alignment) run the generic kernel.
+ * M == 0 or N == 0 is a no-op; K == 0 writes zeros.
+ */
+int neogemm_bf16(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int64_t lda,
+                 int64_t ldb, int64_t ldc, int b_layout, int c_layout, void* workspace,
+                 size_t workspace_bytes, void* hip_stream);
+
+/*
+ * Upper bound of the scratch neogemm_bf16 may use for (M,N,K), in bytes.  Host-only arithmetic.
+ * Counterpart of the per-call device allocations the reference's launcher makes for its TMA
+ * descriptors (v01.cu:153-160, nemgemmV03.cu:60-68): here the caller owns the scratch.
+ */
+size_t neogemm_bf16_workspace_bytes(int64_t M, int64_t N, int64_t K);
+
+/*
+ * Same as neogemm_bf16 but with the kernel variant, the split-K factor (>= 1; 0 = choose) and the
+ * tile-order group height (0 = default) forced.  The reference fixes these at compile time
+ * (template arguments at v01.cu:304-311); this entry point exists for tuning, tests and the bench.
+ * Returns NEOGEMM_ERR_UNSUPPORTED if the variant cannot run the shape.  With split_k > 1 the
+ * workspace must hold split_k * M * N floats.
+ */
+int neogemm_bf16_variant(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K,
+                         int64_t lda, int64_t ldb, int64_t ldc, int b_layout, int c_layout,
+                         void* workspace, size_t workspace_bytes, void* hip_stream, int variant,
+                         int split_k, int group_m);
+
+/*
+ * What neogemm_bf16 would pick for this call: writes the variant id and split-K factor.  Host only.
+ * `aligned` is nonzero when pointers and leading dimensions satisfy the MFMA path (16-byte / 8-element).
+ */
+int neogemm_bf16_plan(int64_t M, int64_t N, int64_t K, int b_layout, int c_layout, int aligned,
+                      int* variant, int* split_k);
+
+/* Text for a status code; replaces the std::cerr print at nemgemmV03.cu:387-390. Never NULL. */
+const char* neogemm_strerror(int status);
+
+/* Library version string, e.g. "neogemm 0.1 gfx950". */
+const char* neogemm_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NEOGEMM_H */
