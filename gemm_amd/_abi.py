@@ -27,6 +27,8 @@ PROTOTYPES = {
     "neogemm_bf16_variant": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _vp, _sz, _vp,
                                     _int, _int, _int]),
     "neogemm_bf16_plan": (_int, [_i64, _i64, _i64, _int, _int, _int, ctypes.POINTER(_int), ctypes.POINTER(_int)]),
+    "neogemm_bf16_profile": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _int, _vp, _int, _int, _vp, _sz]),
+    "neogemm_bf16_profile_bytes": (_sz, [_i64, _i64, _int]),
     "neogemm_strerror": (ctypes.c_char_p, [_int]),
     "neogemm_version": (ctypes.c_char_p, []),
 }

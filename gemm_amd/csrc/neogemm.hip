@@ -12,6 +12,7 @@
 #include <stdio.h>
 
 #include <type_traits>
+#include <utility>
 
 #include "neogemm.h"
 
@@ -27,25 +28,29 @@ typedef __attribute__((ext_vector_type(8))) short i16x8;
 
 #define NEOGEMM_AS3 __attribute__((address_space(3)))
 
-static constexpr int KT = 64;                      // K depth of one LDS stage (bf16 elements)
+static constexpr int KT = 32;                        // K depth of one LDS slab (bf16 elements)
+static constexpr int NSLAB = 4;                      // slabs in the LDS ring
 static constexpr uint32_t OOB_OFFSET = 0x80000000u;  // >= every num_records this file builds
 
 // ---------------------------------------------------------------------------------------------
-// LDS image of an operand tile and its swizzles.
+// LDS image of one operand slab (ROWS x 32 k) and its swizzles.
 //
 // K-major operand (rows of the matrix are K-contiguous: A[M,K], B[N,K]):
-//   image = ROWS x 128 B, row r at r*128, eight 16-byte chunks per row; logical chunk c of row r
-//   lives at physical chunk c ^ swz_k(r).  An MFMA operand read has 32 lanes fetch the same logical
-//   chunk of 32 consecutive rows; swz_k makes any 8 consecutive rows hit 8 distinct chunks and any
-//   16 consecutive rows hit 16 distinct 16-byte slots of a 256-byte window.
+//   image = ROWS x 64 B, row r at r*64, four 16-byte chunks per row; logical chunk c of row r lives
+//   at physical chunk c ^ swz_k(r).  An MFMA operand read has 32 lanes fetch the same logical chunk
+//   of 32 consecutive rows; swz_k makes any 8 consecutive rows cover the 8 slots of a 128-byte
+//   window and any 16 consecutive rows the 16 slots of a 256-byte window exactly once.
 // MN-major operand (the K index is the slow one: B[K,N]):
-//   image = 64 x (ROWS*2) B, k-row at k*ROWS*2; logical chunk c (8 columns) of k-row k lives at
-//   physical chunk c ^ swz_mn(k & 3).  Read back with ds_read_b64_tr_b16, whose 16-lane groups pull
-//   4 k-rows x 16 columns and hand lane j the 4 k-values of column j.
+//   image = 32 x (ROWS*2) B, k-row at k*ROWS*2; logical chunk c (8 columns) of k-row k lives at
+//   physical chunk c ^ swz_mn(k & 3).  Read back with ds_read_b64_tr_b16: in each group of 16 lanes,
+//   lanes 4r..4r+3 address k-row r (16 columns, 8 bytes per lane) and lane j receives the 4 k-values
+//   of column j.
 // Direct-to-LDS loads write 64 lanes x 16 B contiguously, so the swizzle is applied by choosing which
 // global chunk each lane fetches.
 // ---------------------------------------------------------------------------------------------
-__device__ __forceinline__ uint32_t swz_k(uint32_t row) { return ((row >> 1) & 7u) ^ ((row & 1u) << 2); }
+__device__ __forceinline__ uint32_t swz_k(uint32_t row) {
+  return (((row >> 2) & 1u) << 1) | (((row >> 1) ^ (row >> 3)) & 1u);
+}
 __device__ __forceinline__ uint32_t swz_mn(uint32_t k4) {
   // k4 in 0..3 -> {0, 4, 10, 14}
   uint32_t u = (k4 << 1) ^ (k4 >> 1);
@@ -70,6 +75,15 @@ __device__ __forceinline__ i16x4 lds_read_tr16(uint32_t addr) {
   return __builtin_amdgcn_ds_read_tr16_b64_v4i16((NEOGEMM_AS3 i16x4*)(uintptr_t)addr);
 }
 
+template <int N, class Fn, int... I>
+__device__ __forceinline__ void static_for_impl(Fn&& fn, std::integer_sequence<int, I...>) {
+  (fn(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class Fn>
+__device__ __forceinline__ void static_for(Fn&& fn) {
+  static_for_impl<N>(fn, std::make_integer_sequence<int, N>{});
+}
+
 struct TileArgs {
   const char* A;  // operand whose rows become output rows
   const char* B;  // operand whose rows/columns become output columns
@@ -78,17 +92,20 @@ struct TileArgs {
   int M, N, K;
   long lda, ldb, ldc;  // elements
   int ntm, ntn, group_m;
-  int ksplit, ktiles_per_split;
+  int ksplit, ktiles_per_split;  // K is cut in slabs of KT; a split is a run of slabs
+  unsigned long long* prof;      // phase timers, 4 per wave (profiling instantiation only)
 };
 
+// Global -> LDS side of one operand: which 16 bytes each lane fetches for each of this wave's
+// 1 KiB loads of a slab, and the buffer resource that walks along K.
 template <int ROWS, bool KMAJOR, int NW>
 struct Operand {
-  static constexpr int NINSTR = ROWS / 8;        // 1 KiB wave-loads per 64-deep tile
-  static constexpr int IPW = NINSTR / NW;        // per wave
-  static constexpr int ROWB = ROWS * 2;          // bytes per k-row of an MN-major image
-  static constexpr int CPR = ROWS / 8;           // 16-byte chunks per k-row (MN-major)
-  static constexpr int KR = 64 / CPR;            // k-rows per wave-load (MN-major)
-  static_assert(NINSTR % NW == 0, "tile loads must divide evenly over the waves");
+  static constexpr int NINSTR = ROWS / 16;  // 1 KiB wave-loads per slab
+  static constexpr int IPW = NINSTR / NW;   // per wave
+  static constexpr int ROWB = ROWS * 2;     // bytes per k-row of an MN-major image
+  static constexpr int CPR = ROWS / 8;      // 16-byte chunks per k-row (MN-major)
+  static constexpr int KR = 64 / CPR;       // k-rows per wave-load (MN-major)
+  static_assert(NINSTR % NW == 0 && IPW >= 1, "slab loads must divide evenly over the waves");
   static_assert(KMAJOR || ROWS >= 128, "MN-major swizzle needs >= 16 chunks per k-row");
 
   uint32_t voff[IPW];
@@ -104,8 +121,8 @@ struct Operand {
       kadv = KT * 2;
 #pragma unroll
       for (int j = 0; j < IPW; ++j) {
-        uint32_t row = (wave * IPW + j) * 8 + (lane >> 3);
-        uint32_t c = (lane & 7) ^ swz_k(row);
+        uint32_t row = (wave * IPW + j) * 16 + (lane >> 2);
+        uint32_t c = (lane & 3) ^ swz_k(row);
         voff[j] = row * (uint32_t)ld * 2 + c * 16;
       }
     } else {
@@ -124,44 +141,47 @@ struct Operand {
     lds_w = wave * IPW * 1024;
   }
 
-  // K-major only: drop the chunks of the last, partial K tile (they would wrap into the next row).
+  // K-major only: drop the chunks of the last, partial slab (they would wrap into the next row).
+  // An MN-major slab needs nothing: its k-rows past K lie beyond the end of the buffer.
   __device__ __forceinline__ void mask_k_tail(int krem, int wave, int lane) {
     if constexpr (KMAJOR) {
 #pragma unroll
       for (int j = 0; j < IPW; ++j) {
-        uint32_t row = (wave * IPW + j) * 8 + (lane >> 3);
-        uint32_t c = (lane & 7) ^ swz_k(row);
+        uint32_t row = (wave * IPW + j) * 16 + (lane >> 2);
+        uint32_t c = (lane & 3) ^ swz_k(row);
         if ((int)c * 8 >= krem) voff[j] = OOB_OFFSET;
       }
     }
   }
 
-  __device__ __forceinline__ void issue(uint32_t lds_tile) const {
+  __device__ __forceinline__ i32x4 rsrc() const {
     const uint64_t rem = end - base;
     const uint32_t nr = (rem >> 31) ? 0x80000000u : (uint32_t)rem;
-    i32x4 rsrc;
-    rsrc[0] = (int)(uint32_t)base;
-    rsrc[1] = (int)((uint32_t)(base >> 32) & 0xffffu);
-    rsrc[2] = (int)nr;
-    rsrc[3] = 0x00020000;
-#pragma unroll
-    for (int j = 0; j < IPW; ++j) dma16(rsrc, lds_tile + lds_w + j * 1024, voff[j]);
+    i32x4 r;
+    r[0] = (int)(uint32_t)base;
+    r[1] = (int)((uint32_t)(base >> 32) & 0xffffu);
+    r[2] = (int)nr;
+    r[3] = 0x00020000;
+    return r;
+  }
+  __device__ __forceinline__ void issue_one(i32x4 r, uint32_t lds_img, int j) const {
+    dma16(r, lds_img + lds_w + j * 1024, voff[j]);
   }
   __device__ __forceinline__ void advance() { base += kadv; }
 };
 
-// Per-lane constants for reading MFMA operand fragments (32 rows x 16 k per fragment) out of the image.
+// Per-lane constants for reading MFMA operand fragments (32 rows x 16 k per fragment) out of a slab image.
 template <int ROWS, bool KMAJOR, int NT>
 struct FragReader {
   static constexpr int ROWB = ROWS * 2;
   uint32_t lane_off[KMAJOR ? 1 : NT];
-  uint32_t xs[KMAJOR ? 4 : 1];
+  uint32_t xs[KMAJOR ? 2 : 1];
 
   __device__ __forceinline__ void init(int wrow0, int lane) {
     if constexpr (KMAJOR) {
-      lane_off[0] = (uint32_t)(wrow0 + (lane & 31)) * 128;
+      lane_off[0] = (uint32_t)(wrow0 + (lane & 31)) * 64;
 #pragma unroll
-      for (int s = 0; s < 4; ++s) xs[s] = (((uint32_t)(2 * s + (lane >> 5))) ^ swz_k(lane & 15)) << 4;
+      for (int s = 0; s < 2; ++s) xs[s] = (((uint32_t)(2 * s + (lane >> 5))) ^ swz_k(lane & 15)) << 4;
     } else {
       const uint32_t i = lane & 15, g1 = (lane >> 4) & 1, h = lane >> 5;
       const uint32_t tr_r = i >> 2, tr_c = i & 3;
@@ -173,10 +193,10 @@ struct FragReader {
       xs[0] = 0;
     }
   }
-  // fragment t (32 rows), k-step s (16 deep) of the tile image at LDS address `img`
+  // fragment t (32 rows), k-step s (16 deep, 0 or 1) of the slab image at LDS address `img`
   __device__ __forceinline__ bf16x8 read(uint32_t img, int t, int s) const {
     if constexpr (KMAJOR) {
-      return lds_read_b128(img + lane_off[0] + t * 4096 + xs[s]);
+      return lds_read_b128(img + lane_off[0] + t * 2048 + xs[s]);
     } else {
       i16x4 lo = lds_read_tr16(img + lane_off[t] + (16 * s) * ROWB);
       i16x4 hi = lds_read_tr16(img + lane_off[t] + (16 * s + 4) * ROWB);
@@ -186,13 +206,19 @@ struct FragReader {
   }
 };
 
-template <int BM, int BN, int WGM, int WGN, bool AK, bool BK>
+// PROF adds s_memtime stamps around the two waits of the main loop and writes, per wave,
+// {total, waiting for own loads, waiting at the barrier, epilogue} shader-clock cycles to p.prof — the
+// per-phase cycle buffer idea of the reference's harness (cublass/matmul.cu:99-106,149-165).
+template <int BM, int BN, int WGM, int WGN, bool AK, bool BK, bool PROF = false>
 __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
   constexpr int NW = WGM * WGN;
   constexpr int WTM = BM / WGM, WTN = BN / WGN;
   constexpr int TM = WTM / 32, TN = WTN / 32;
-  constexpr uint32_t A_BYTES = BM * 128, B_BYTES = BN * 128, STAGE = A_BYTES + B_BYTES;
+  constexpr uint32_t A_BYTES = BM * KT * 2, B_BYTES = BN * KT * 2, SLAB = A_BYTES + B_BYTES;
   static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be a multiple of the 32x32 MFMA tile");
+  using OpA = Operand<BM, AK, NW>;
+  using OpB = Operand<BN, BK, NW>;
+  constexpr int LA = OpA::IPW, LB = OpB::IPW, LPS = LA + LB;  // this wave's loads per slab
 
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   const uint32_t lds0 = (uint32_t)(uintptr_t)(NEOGEMM_AS3 char*)smem;
@@ -221,11 +247,14 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
   const int k_begin = kz * p.ktiles_per_split * KT;
   int k_end = k_begin + p.ktiles_per_split * KT;
   if (k_end > p.K) k_end = p.K;
-  const int nkt = (k_end - k_begin + KT - 1) / KT;
-  const int k_tail = (k_end - k_begin) - (nkt - 1) * KT;  // depth of the last tile, 1..64
+  const int nslab = (k_end - k_begin + KT - 1) / KT;
+  const int k_tail = (k_end - k_begin) - (nslab - 1) * KT;  // depth of the last slab, 1..KT
 
-  Operand<BM, AK, NW> opa;
-  Operand<BN, BK, NW> opb;
+  unsigned long long t_start = 0, t_loads = 0, t_barrier = 0;
+  if constexpr (PROF) t_start = __builtin_readcyclecounter();
+
+  OpA opa;
+  OpB opb;
   opa.init(p.A, p.lda, p.M, m0, k_begin, p.K, wave, lane);
   opb.init(p.B, p.ldb, p.N, n0, k_begin, p.K, wave, lane);
   FragReader<BM, AK, TM> fa;
@@ -241,86 +270,153 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-  // tail_check: the tile being loaded may be the last, partial one (never true in the steady loop)
-  auto load_tile = [&](int kt, uint32_t stage, bool tail_check) {
-    if (tail_check && kt == nkt - 1 && k_tail != KT) {
+  bf16x8 af[2][TM], bfr[2][TN];
+
+  // One k-step (16 deep): the MFMAs of fragment buffer `cur`, the LDS reads that fill the other
+  // buffer from slab image `img_next` / k-step `s_next`, and this wave's loads of one operand of a
+  // later slab into image `img_dma`.  The work is cut into groups — one direct-to-LDS load per group,
+  // the LDS reads in the first half of the groups — so that the wave never issues a burst of memory
+  // instructions: a burst backs up the vector-memory queue and the wave, which issues in order,
+  // cannot reach its next MFMA until the queue has drained.
+  auto kstep = [&](int cur, auto do_read, uint32_t img_next, int s_next, auto dma_a, auto dma_b, uint32_t img_dma) {
+    constexpr bool READ = decltype(do_read)::value;
+    constexpr bool DMA_A = decltype(dma_a)::value, DMA_B = decltype(dma_b)::value;
+    constexpr int NL = DMA_A ? LA : (DMA_B ? LB : 0);
+    constexpr int NG = NL > 0 ? (NL < TM * TN ? NL : TM * TN) : 2;   // groups
+    constexpr int MPG = (TM * TN) / NG;                              // MFMAs per group
+    static_assert((TM * TN) % NG == 0, "MFMAs must divide over the groups");
+    constexpr int RG = NG >= 2 ? NG / 2 : 1;                          // groups that carry LDS reads
+    constexpr int NFRAG = TM + TN;
+    constexpr int FPG = (NFRAG + RG - 1) / RG;                        // fragments read per group
+    i32x4 rs;
+    if constexpr (DMA_A) rs = opa.rsrc();
+    if constexpr (DMA_B) rs = opb.rsrc();
+    static_for<NG>([&](auto gc) {
+      constexpr int g = decltype(gc)::value;
+      constexpr int f0 = g * FPG, f1 = (g + 1) * FPG < NFRAG ? (g + 1) * FPG : NFRAG;
+      constexpr bool READS = READ && g < RG && f0 < f1;
+      // LDS read instructions this group issues (an MN-major fragment takes two transposing reads)
+      constexpr int na = READS ? ((f1 < TM ? f1 : TM) - (f0 < TM ? f0 : TM)) : 0;
+      constexpr int nb = READS ? ((f1 - f0) - na) : 0;
+      constexpr int nread = na * (AK ? 1 : 2) + nb * (BK ? 1 : 2);
+      if constexpr (READS) {
+#pragma unroll
+        for (int f = f0; f < f1; ++f) {
+          if (f < TM) af[cur ^ 1][f] = fa.read(img_next, f, s_next);
+          else bfr[cur ^ 1][f - TM] = fb.read(img_next + A_BYTES, f - TM, s_next);
+        }
+      }
+#pragma unroll
+      for (int m = g * MPG; m < (g + 1) * MPG; ++m) {
+        const int i = m / TN, j = m % TN;
+        // B fragment first: D rows index n, D columns index m, so a lane ends up with 4
+        // consecutive n of one output row (an 8-byte store) instead of 4 rows of one column.
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[cur][j], af[cur][i], acc[i][j], 0, 0, 0);
+      }
+      // within the group: one MFMA first, then the LDS reads, then the rest of the MFMAs
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      if constexpr (nread > 0) __builtin_amdgcn_sched_group_barrier(0x100, nread, 0);
+      if constexpr (MPG > 1) __builtin_amdgcn_sched_group_barrier(0x008, MPG - 1, 0);
+      if constexpr (NL > 0) {
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (DMA_A) {
+          if constexpr (g < LA) opa.issue_one(rs, img_dma, g);
+        } else {
+          if constexpr (g < LB) opb.issue_one(rs, img_dma + A_BYTES, g);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    });
+    if constexpr (DMA_A) opa.advance();
+    if constexpr (DMA_B) opb.advance();
+  };
+
+  auto img_of = [&](int slab) -> uint32_t { return lds0 + (uint32_t)(slab & (NSLAB - 1)) * SLAB; };
+  auto load_slab_burst = [&](int j) {
+    if (j == nslab - 1 && k_tail != KT) {
       opa.mask_k_tail(k_tail, wave, lane);
       opb.mask_k_tail(k_tail, wave, lane);
     }
-    opa.issue(lds0 + stage * STAGE);
-    opb.issue(lds0 + stage * STAGE + A_BYTES);
+    const i32x4 ra = opa.rsrc(), rb = opb.rsrc();
+#pragma unroll
+    for (int i = 0; i < LA; ++i) opa.issue_one(ra, img_of(j), i);
+#pragma unroll
+    for (int i = 0; i < LB; ++i) opb.issue_one(rb, img_of(j) + A_BYTES, i);
     opa.advance();
     opb.advance();
   };
-
-  bf16x8 af[2][TM], bfr[2][TN];
-  auto read_frags = [&](int buf, uint32_t stage, int s) {
-    const uint32_t imgA = lds0 + stage * STAGE, imgB = imgA + A_BYTES;
-#pragma unroll
-    for (int t = 0; t < TM; ++t) af[buf][t] = fa.read(imgA, t, s);
-#pragma unroll
-    for (int t = 0; t < TN; ++t) bfr[buf][t] = fb.read(imgB, t, s);
-  };
-  auto mfma_step = [&](int buf) {
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-      for (int j = 0; j < TN; ++j)
-        // B fragment first: D rows index n, D columns index m, so a lane ends up with 4
-        // consecutive n of one output row (an 8-byte store) instead of 4 rows of one column.
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[buf][j], af[buf][i], acc[i][j], 0, 0, 0);
-  };
-  // LDS reads of the next k-step are issued two per MFMA at the head of the current step.
-  constexpr int NREAD = TM * (AK ? 1 : 2) + TN * (BK ? 1 : 2);
-  auto sched_step = [&]() {
-#pragma unroll
-    for (int i = 0; i < (NREAD + 1) / 2; ++i) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
-      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // 2 DS reads
-    }
-    __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - (NREAD + 1) / 2, 0);
-  };
-
-  // One 64-deep K tile = 4 k-steps.  Fragments of step s+1 are fetched under the MFMAs of step s,
-  // across tile boundaries too: before the last step of a tile every wave waits for its own loads of
-  // the next tile and meets the others at the barrier; past it the next tile is readable everywhere
-  // and the current tile's image is dead (its last fragments are already in registers), so the tile
-  // after next is streamed into it while the last step's MFMAs run.
-  auto tile_body = [&](int kt, uint32_t stage, auto steady, bool has_next, bool has_next2) {
-    read_frags(1, stage, 1);
-    mfma_step(0);
-    sched_step();
-    read_frags(0, stage, 2);
-    mfma_step(1);
-    sched_step();
-    read_frags(1, stage, 3);
-    mfma_step(0);
-    sched_step();
-    if (decltype(steady)::value || has_next) {
-      __builtin_amdgcn_sched_barrier(0);  // keep step 2's MFMAs above the wait
-      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+  // Wait until this wave's loads of the slab about to be read have landed (all but the `keep` most
+  // recent loads), and its own LDS reads are done; then meet the other waves.
+  auto sync = [&](auto keep) {
+    constexpr int KEEP = decltype(keep)::value;
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (PROF) {
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      const unsigned long long t0 = __builtin_readcyclecounter();
+      asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(KEEP), "s"(t0) : "memory");
+      const unsigned long long t1 = __builtin_readcyclecounter();
+      asm volatile("s_waitcnt lgkmcnt(0)" ::"s"(t1) : "memory");
       __builtin_amdgcn_s_barrier();
-      asm volatile("" ::: "memory");
-      if (decltype(steady)::value || has_next2) load_tile(kt + 2, stage, !decltype(steady)::value);
-      __builtin_amdgcn_sched_barrier(0);
-      read_frags(0, stage ^ 1, 0);
+      const unsigned long long t2 = __builtin_readcyclecounter();
+      asm volatile("s_waitcnt lgkmcnt(0)" ::"s"(t2) : "memory");
+      t_loads += t1 - t0;
+      t_barrier += t2 - t1;
+    } else {
+      asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(KEEP) : "memory");
+      __builtin_amdgcn_s_barrier();
     }
-    mfma_step(1);
-    sched_step();
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
   };
+  using T = std::true_type;
+  using F = std::false_type;
 
-  load_tile(0, 0, true);
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  __builtin_amdgcn_s_barrier();
-  asm volatile("" ::: "memory");
-  if (nkt > 1) load_tile(1, 1, true);
-  read_frags(0, 0, 0);
-  int kt = 0;
-  for (; kt + 4 < nkt; kt += 2) {  // the tile loaded by the second body (kt + 3) is never the last
-    tile_body(kt, 0, std::true_type{}, true, true);
-    tile_body(kt + 1, 1, std::true_type{}, true, true);
+  // Ring of NSLAB slab images; slab j lives in image j % NSLAB.  Steady state, for slab j:
+  //   k-step 0 of slab j    reads the fragments of k-step 1 of slab j
+  //   sync                  all waves are done reading slab j, slab j+1 has landed everywhere
+  //   k-step 1 of slab j    reads k-step 0 of slab j+1, streams the A part of slab j+4 into image j%4
+  //   k-step 0 of slab j+1  reads k-step 1 of slab j+1, streams the B part of slab j+4
+  // so a load has at least two slab-times to land and loads leave the wave one at a time.
+  {
+    const int npre = nslab < NSLAB ? nslab : NSLAB;
+    for (int j = 0; j < npre; ++j) load_slab_burst(j);
+    // slab 0 landed: everything but the later slabs' loads
+    if (npre == 4) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * LPS) : "memory");
+    else if (npre == 3) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * LPS) : "memory");
+    else if (npre == 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LPS) : "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
   }
-  for (; kt < nkt; ++kt) tile_body(kt, kt & 1, std::false_type{}, kt + 1 < nkt, kt + 2 < nkt);
+#pragma unroll
+  for (int t = 0; t < TM; ++t) af[0][t] = fa.read(img_of(0), t, 0);
+#pragma unroll
+  for (int t = 0; t < TN; ++t) bfr[0][t] = fb.read(img_of(0) + A_BYTES, t, 0);
+  kstep(0, T{}, img_of(0), 1, F{}, F{}, 0);
+
+  int j = 0;
+  // steady: slab j+4 exists and is not the last one (the last may need its K tail masked)
+  for (; j + 3 + NSLAB < nslab - 1; j += NSLAB) {
+#pragma unroll
+    for (int u = 0; u < NSLAB; ++u) {
+      const uint32_t img_free = lds0 + u * SLAB, img_next = lds0 + ((u + 1) & (NSLAB - 1)) * SLAB;
+      sync(std::integral_constant<int, 2 * LPS>{});
+      kstep(1, T{}, img_next, 0, T{}, F{}, img_free);
+      kstep(0, T{}, img_next, 1, F{}, T{}, img_free);
+    }
+  }
+  // tail: runtime slab indices, loads in a burst, conservative waits
+  for (; j + 1 < nslab; ++j) {
+    sync(std::integral_constant<int, 0>{});
+    if (j + NSLAB < nslab) load_slab_burst(j + NSLAB);
+    kstep(1, T{}, img_of(j + 1), 0, F{}, F{}, 0);
+    kstep(0, T{}, img_of(j + 1), 1, F{}, F{}, 0);
+  }
+  kstep(1, F{}, 0, 0, F{}, F{}, 0);
+  // every load was waited for by the last sync (or the prologue when there is one slab)
+
+  unsigned long long t_main = 0;
+  if constexpr (PROF) t_main = __builtin_readcyclecounter();
 
   // Epilogue: lane holds, per 32x32 tile, output row (lane & 31) and four runs of 4 consecutive columns.
   const int row_l = lane & 31, colq = (lane >> 5) * 4;
@@ -371,6 +467,17 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
           }
         }
       }
+    }
+  }
+  if constexpr (PROF) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    const unsigned long long t_end = __builtin_readcyclecounter();
+    if (lane == 0 && p.prof) {
+      unsigned long long* o = p.prof + ((size_t)blockIdx.x * NW + wave) * 4;
+      o[0] = t_end - t_start;
+      o[1] = t_loads;
+      o[2] = t_barrier;
+      o[3] = t_end - t_main;
     }
   }
 }
@@ -437,7 +544,7 @@ static const VariantInfo kVariants[NEOGEMM_VARIANT_COUNT] = {
 
 template <int BM, int BN, int WGM, int WGN>
 static hipError_t launch_tile(const TileArgs& a, bool ak, bool bk, hipStream_t st) {
-  constexpr size_t lds = 2 * (size_t)(BM + BN) * 128;
+  constexpr size_t lds = (size_t)NSLAB * (BM + BN) * KT * 2;
   dim3 grid(a.ntm * a.ntn, a.ksplit), block(WGM * WGN * 64);
   auto go = [&](auto kern) -> hipError_t {
     static bool attr_done = false;  // per instantiation
@@ -449,6 +556,13 @@ static hipError_t launch_tile(const TileArgs& a, bool ak, bool bk, hipStream_t s
     kern<<<grid, block, lds, st>>>(a);
     return hipGetLastError();
   };
+  if (a.prof) {
+    if constexpr (BM == 256 && BN == 256) {
+      if (ak && bk) return go(gemm_tile_kernel<BM, BN, WGM, WGN, true, true, true>);
+      if (ak && !bk) return go(gemm_tile_kernel<BM, BN, WGM, WGN, true, false, true>);
+    }
+    return hipErrorInvalidValue;
+  }
   if (ak && bk) return go(gemm_tile_kernel<BM, BN, WGM, WGN, true, true>);
   if (ak && !bk) {
     if constexpr (BN >= 128) return go(gemm_tile_kernel<BM, BN, WGM, WGN, true, false>);
@@ -494,7 +608,7 @@ static void plan(int64_t M, int64_t N, int64_t K, bool aligned, int* variant, in
 
 static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
                int64_t ldc, int b_layout, int c_layout, void* workspace, size_t workspace_bytes, void* hip_stream,
-               int variant, int split_k, int group_m) {
+               int variant, int split_k, int group_m, unsigned long long* prof = nullptr) {
   if (M < 0 || N < 0 || K < 0) return NEOGEMM_ERR_BAD_ARG;
   if ((b_layout != NEOGEMM_B_KN && b_layout != NEOGEMM_B_NK) || (c_layout != NEOGEMM_C_ROW && c_layout != NEOGEMM_C_COL))
     return NEOGEMM_ERR_BAD_ARG;
@@ -559,6 +673,8 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
   a.ktiles_per_split = ceil_div(ktiles, s);
   a.ksplit = ceil_div(ktiles, a.ktiles_per_split);  // no empty split
   a.ws = nullptr;
+  a.prof = prof;
+  if (prof && (a.ksplit > 1 || vi.bm != 256 || vi.bn != 256 || !ak)) return NEOGEMM_ERR_UNSUPPORTED;
   if (a.ksplit > 1) {
     const size_t need = (size_t)a.ksplit * (size_t)M * (size_t)N * sizeof(float);
     if (!workspace || workspace_bytes < need) return NEOGEMM_ERR_WORKSPACE;
@@ -607,6 +723,22 @@ int neogemm_bf16_variant(const void* A, const void* B, void* C, int64_t M, int64
                          size_t workspace_bytes, void* hip_stream, int variant, int split_k, int group_m) {
   return neogemm::run(A, B, C, M, N, K, lda, ldb, ldc, b_layout, c_layout, workspace, workspace_bytes, hip_stream,
                       variant, split_k, group_m);
+}
+
+int neogemm_bf16_profile(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int64_t lda,
+                         int64_t ldb, int64_t ldc, int b_layout, void* hip_stream, int variant, int group_m,
+                         unsigned long long* phase_cycles, size_t phase_cycles_bytes) {
+  if (!phase_cycles) return NEOGEMM_ERR_BAD_ARG;
+  if (variant != NEOGEMM_VARIANT_T256x256_W8 && variant != NEOGEMM_VARIANT_T256x256_W4) return NEOGEMM_ERR_UNSUPPORTED;
+  if (phase_cycles_bytes < neogemm_bf16_profile_bytes(M, N, variant)) return NEOGEMM_ERR_WORKSPACE;
+  return neogemm::run(A, B, C, M, N, K, lda, ldb, ldc, b_layout, NEOGEMM_C_ROW, nullptr, 0, hip_stream, variant, 1,
+                      group_m, phase_cycles);
+}
+
+size_t neogemm_bf16_profile_bytes(int64_t M, int64_t N, int variant) {
+  if (M <= 0 || N <= 0) return 0;
+  const int waves = variant == NEOGEMM_VARIANT_T256x256_W4 ? 4 : 8;
+  return (size_t)neogemm::ceil_div(M, 256) * neogemm::ceil_div(N, 256) * waves * 4 * sizeof(unsigned long long);
 }
 
 size_t neogemm_bf16_workspace_bytes(int64_t M, int64_t N, int64_t K) {

@@ -1,0 +1,240 @@
+// Stand-alone timing harness: hipBLASLt and rocBLAS beside libneogemm on the same device buffers.
+//
+// Takes the role of the reference's cuBLAS harness (cublass/matmul.cu:82-196: N(0,1) host init,
+// cublasGemmEx bf16 with fp32 compute :33-43, event-timed repetitions :169-183, TFLOPS print) with
+// the vendor libraries of this platform.  Unlike the reference it takes the shape from the command
+// line, handles non-square shapes (the reference's lda/ldc only work for squares, matmul.cu:36-37),
+// scales the inputs by 1/sqrt(K), rotates the weight buffer for shapes whose working set fits the
+// last-level cache, and cross-checks the libraries against each other.
+//
+//   matmul_bench M N K [reps=100] [b_layout=0|1] [variant=0] [split_k=0] [group_m=0] [nbuf=1]
+//
+// One line of JSON per library on stdout.
+#include <hip/hip_runtime.h>
+#include <hipblaslt/hipblaslt.h>
+#include <rocblas/rocblas.h>
+
+#include <algorithm>
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <random>
+#include <vector>
+
+#include "neogemm.h"
+
+#define HIP_OK(x)                                                                          \
+  do {                                                                                     \
+    hipError_t e_ = (x);                                                                   \
+    if (e_ != hipSuccess) {                                                                \
+      fprintf(stderr, "%s:%d %s -> %s\n", __FILE__, __LINE__, #x, hipGetErrorString(e_)); \
+      exit(1);                                                                             \
+    }                                                                                      \
+  } while (0)
+#define BLT_OK(x)                                                          \
+  do {                                                                     \
+    hipblasStatus_t s_ = (x);                                              \
+    if (s_ != HIPBLAS_STATUS_SUCCESS) {                                    \
+      fprintf(stderr, "%s:%d %s -> %d\n", __FILE__, __LINE__, #x, (int)s_); \
+      exit(1);                                                             \
+    }                                                                      \
+  } while (0)
+
+static uint16_t f2bf(float f) {
+  uint32_t u;
+  memcpy(&u, &f, 4);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+static float bf2f(uint16_t h) {
+  uint32_t u = (uint32_t)h << 16;
+  float f;
+  memcpy(&f, &u, 4);
+  return f;
+}
+
+template <class F>
+static double time_ms(F&& launch, int reps, hipStream_t st) {
+  hipEvent_t a, b;
+  HIP_OK(hipEventCreate(&a));
+  HIP_OK(hipEventCreate(&b));
+  const int warm = std::max(3, reps / 10);
+  for (int i = 0; i < warm; ++i) launch(i);
+  HIP_OK(hipStreamSynchronize(st));
+  // median of 5 batches
+  std::vector<double> ms;
+  for (int batch = 0; batch < 5; ++batch) {
+    HIP_OK(hipEventRecord(a, st));
+    for (int i = 0; i < reps; ++i) launch(i);
+    HIP_OK(hipEventRecord(b, st));
+    HIP_OK(hipEventSynchronize(b));
+    float t;
+    HIP_OK(hipEventElapsedTime(&t, a, b));
+    ms.push_back(t / reps);
+  }
+  std::sort(ms.begin(), ms.end());
+  HIP_OK(hipEventDestroy(a));
+  HIP_OK(hipEventDestroy(b));
+  return ms[ms.size() / 2];
+}
+
+static void report(const char* lib, int64_t M, int64_t N, int64_t K, int bl, double ms, const char* extra) {
+  const double flop = 2.0 * M * N * K, bytes = 2.0 * (M * K + K * N + M * N);
+  printf("{\"lib\": \"%s\", \"M\": %lld, \"N\": %lld, \"K\": %lld, \"b_layout\": %d, \"ms\": %.5f, \"tflops\": %.2f, "
+         "\"pct_of_2500\": %.2f, \"gbps\": %.1f, \"pct_of_8000\": %.2f%s}\n",
+         lib, (long long)M, (long long)N, (long long)K, bl, ms, flop / ms / 1e9, flop / ms / 1e9 / 25.0,
+         bytes / ms / 1e6, bytes / ms / 1e6 / 80.0, extra);
+  fflush(stdout);
+}
+
+int main(int argc, char** argv) {
+  if (argc < 4) {
+    fprintf(stderr, "usage: %s M N K [reps] [b_layout] [variant] [split_k] [group_m] [nbuf]\n", argv[0]);
+    return 2;
+  }
+  const int64_t M = atoll(argv[1]), N = atoll(argv[2]), K = atoll(argv[3]);
+  const int reps = argc > 4 ? atoi(argv[4]) : 100;
+  const int bl = argc > 5 ? atoi(argv[5]) : 0;
+  const int variant = argc > 6 ? atoi(argv[6]) : 0;
+  const int split_k = argc > 7 ? atoi(argv[7]) : 0;
+  const int group_m = argc > 8 ? atoi(argv[8]) : 0;
+  const int nbuf = argc > 9 ? std::max(1, atoi(argv[9])) : 1;
+  const bool only_ours = getenv("NEOGEMM_ONLY") != nullptr;
+
+  hipStream_t st;
+  HIP_OK(hipStreamCreate(&st));
+
+  // N(0,1)/sqrt(K) inputs (cf. matmul.cu:53-59, which leaves them unscaled)
+  std::mt19937 rng(69);
+  std::normal_distribution<float> nd(0.f, 1.f);
+  const float sc = 1.0f / std::sqrt((float)K);
+  std::vector<uint16_t> hA((size_t)M * K), hB((size_t)K * N);
+  for (auto& v : hA) v = f2bf(nd(rng) * sc);
+  for (auto& v : hB) v = f2bf(nd(rng) * sc);  // stored as given: [K,N] for b_layout 0, [N,K] for 1
+  if (getenv("NEOGEMM_ZERO_INPUTS")) {  // power experiment only: zeros switch far fewer wires
+    std::fill(hA.begin(), hA.end(), 0);
+    std::fill(hB.begin(), hB.end(), 0);
+  }
+  void *dA, *dC, *dC2;
+  std::vector<void*> dB(nbuf);
+  HIP_OK(hipMalloc(&dA, hA.size() * 2));
+  HIP_OK(hipMalloc(&dC, (size_t)M * N * 2));
+  HIP_OK(hipMalloc(&dC2, (size_t)M * N * 2));
+  HIP_OK(hipMemcpy(dA, hA.data(), hA.size() * 2, hipMemcpyHostToDevice));
+  for (int i = 0; i < nbuf; ++i) {
+    HIP_OK(hipMalloc(&dB[i], hB.size() * 2));
+    HIP_OK(hipMemcpy(dB[i], hB.data(), hB.size() * 2, hipMemcpyHostToDevice));
+  }
+  const int64_t ldb = bl == 0 ? N : K;
+
+  // ---- libneogemm
+  size_t ws_bytes = neogemm_bf16_workspace_bytes(M, N, K);
+  if (split_k > 1) ws_bytes = std::max(ws_bytes, (size_t)split_k * M * N * 4);
+  void* ws = nullptr;
+  if (ws_bytes) HIP_OK(hipMalloc(&ws, ws_bytes));
+  int pv = 0, ps = 0;
+  neogemm_bf16_plan(M, N, K, bl, 0, 1, &pv, &ps);
+  auto ours = [&](int i) {
+    int s = neogemm_bf16_variant(dA, dB[i % nbuf], dC, M, N, K, K, ldb, N, bl, NEOGEMM_C_ROW, ws, ws_bytes, st,
+                                 variant, split_k, group_m);
+    if (s != NEOGEMM_OK) {
+      fprintf(stderr, "neogemm: %s\n", neogemm_strerror(s));
+      exit(1);
+    }
+  };
+  {
+    double ms = time_ms(ours, reps, st);
+    char extra[128];
+    snprintf(extra, sizeof extra, ", \"variant\": %d, \"split_k\": %d, \"group_m\": %d", variant ? variant : pv,
+             split_k ? split_k : ps, group_m);
+    report("neogemm", M, N, K, bl, ms, extra);
+  }
+  if (only_ours) return 0;
+
+  // ---- hipBLASLt: row-major C[M,N] = A.B is column-major C'[N,M] = op(B') . A'
+  hipblasLtHandle_t lt;
+  BLT_OK(hipblasLtCreate(&lt));
+  hipblasLtMatmulDesc_t desc;
+  BLT_OK(hipblasLtMatmulDescCreate(&desc, HIPBLAS_COMPUTE_32F, HIP_R_32F));
+  hipblasOperation_t opB = bl == 0 ? HIPBLAS_OP_N : HIPBLAS_OP_T, opA = HIPBLAS_OP_N;
+  BLT_OK(hipblasLtMatmulDescSetAttribute(desc, HIPBLASLT_MATMUL_DESC_TRANSA, &opB, sizeof opB));
+  BLT_OK(hipblasLtMatmulDescSetAttribute(desc, HIPBLASLT_MATMUL_DESC_TRANSB, &opA, sizeof opA));
+  hipblasLtMatrixLayout_t lB, lA, lC;
+  if (bl == 0) BLT_OK(hipblasLtMatrixLayoutCreate(&lB, HIP_R_16BF, N, K, N));
+  else BLT_OK(hipblasLtMatrixLayoutCreate(&lB, HIP_R_16BF, K, N, K));
+  BLT_OK(hipblasLtMatrixLayoutCreate(&lA, HIP_R_16BF, K, M, K));
+  BLT_OK(hipblasLtMatrixLayoutCreate(&lC, HIP_R_16BF, N, M, N));
+  hipblasLtMatmulPreference_t pref;
+  BLT_OK(hipblasLtMatmulPreferenceCreate(&pref));
+  size_t lt_ws_bytes = 256ull << 20;
+  void* lt_ws;
+  HIP_OK(hipMalloc(&lt_ws, lt_ws_bytes));
+  BLT_OK(hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &lt_ws_bytes,
+                                               sizeof lt_ws_bytes));
+  const int want = 8;
+  hipblasLtMatmulHeuristicResult_t res[want];
+  int found = 0;
+  BLT_OK(hipblasLtMatmulAlgoGetHeuristic(lt, desc, lB, lA, lC, lC, pref, want, res, &found));
+  const float alpha = 1.f, beta = 0.f;
+  double best = 1e30;
+  int best_i = -1;
+  for (int a = 0; a < found; ++a) {
+    auto fn = [&](int i) {
+      BLT_OK(hipblasLtMatmul(lt, desc, &alpha, dB[i % nbuf], lB, dA, lA, &beta, dC2, lC, dC2, lC, &res[a].algo, lt_ws,
+                             lt_ws_bytes, st));
+    };
+    double ms = time_ms(fn, std::max(10, reps / 4), st);
+    if (ms < best) best = ms, best_i = a;
+  }
+  if (best_i >= 0) {
+    auto fn = [&](int i) {
+      BLT_OK(hipblasLtMatmul(lt, desc, &alpha, dB[i % nbuf], lB, dA, lA, &beta, dC2, lC, dC2, lC, &res[best_i].algo,
+                             lt_ws, lt_ws_bytes, st));
+    };
+    double ms = time_ms(fn, reps, st);
+    char extra[96];
+    snprintf(extra, sizeof extra, ", \"algo_rank\": %d, \"algos_tried\": %d", best_i, found);
+    report("hipblaslt", M, N, K, bl, ms, extra);
+  } else {
+    fprintf(stderr, "hipblaslt: no algorithm found\n");
+  }
+
+  // ---- rocBLAS gemm_ex
+  {
+    rocblas_handle rb;
+    if (rocblas_create_handle(&rb) == rocblas_status_success) {
+      rocblas_set_stream(rb, st);
+      auto fn = [&](int i) {
+        rocblas_gemm_ex(rb, bl == 0 ? rocblas_operation_none : rocblas_operation_transpose, rocblas_operation_none,
+                        (rocblas_int)N, (rocblas_int)M, (rocblas_int)K, &alpha, dB[i % nbuf], rocblas_datatype_bf16_r,
+                        (rocblas_int)ldb, dA, rocblas_datatype_bf16_r, (rocblas_int)K, &beta, dC2,
+                        rocblas_datatype_bf16_r, (rocblas_int)N, dC2, rocblas_datatype_bf16_r, (rocblas_int)N,
+                        rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0);
+      };
+      double ms = time_ms(fn, reps, st);
+      report("rocblas", M, N, K, bl, ms, "");
+      rocblas_destroy_handle(rb);
+    }
+  }
+
+  // ---- cross-check ours against the vendor result left in dC2 (cf. matmul.cu:61-75, abs 0.1 there)
+  {
+    ours(0);
+    HIP_OK(hipStreamSynchronize(st));
+    std::vector<uint16_t> c1((size_t)M * N), c2((size_t)M * N);
+    HIP_OK(hipMemcpy(c1.data(), dC, c1.size() * 2, hipMemcpyDeviceToHost));
+    HIP_OK(hipMemcpy(c2.data(), dC2, c2.size() * 2, hipMemcpyDeviceToHost));
+    double num = 0, den = 0, maxabs = 0;
+    for (size_t i = 0; i < c1.size(); ++i) {
+      double a = bf2f(c1[i]), b = bf2f(c2[i]);
+      num += (a - b) * (a - b);
+      den += b * b;
+      maxabs = std::max(maxabs, std::fabs(a - b));
+    }
+    printf("{\"check\": \"neogemm_vs_vendor\", \"rel_fro\": %.3e, \"max_abs\": %.3e}\n", std::sqrt(num / std::max(den, 1e-300)),
+           maxabs);
+  }
+  return 0;
+}

@@ -95,6 +95,20 @@ int neogemm_bf16_variant(const void* A, const void* B, void* C, int64_t M, int64
 int neogemm_bf16_plan(int64_t M, int64_t N, int64_t K, int b_layout, int c_layout, int aligned,
                       int* variant, int* split_k);
 
+/*
+ * Instrumented run of a 256x256 variant (row-major C, no split-K): besides computing C, every wave
+ * writes four shader-clock cycle counts {whole kernel, waiting for its own global->LDS loads, waiting
+ * at the workgroup barrier, epilogue} to phase_cycles[(workgroup * waves + wave) * 4 + i], with
+ * waves = 8 or 4 by variant and workgroup = launch order.  This is the per-phase cycle buffer of the
+ * reference's harness (the `DB` array: cublass/matmul.cu:99-106 allocation, :149-165 decode), which
+ * no kernel in the reference fills in.  phase_cycles is device memory of at least
+ * neogemm_bf16_profile_bytes(M, N, variant) bytes.  The timers cost a few percent; never time with it.
+ */
+int neogemm_bf16_profile(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int64_t lda,
+                         int64_t ldb, int64_t ldc, int b_layout, void* hip_stream, int variant, int group_m,
+                         unsigned long long* phase_cycles, size_t phase_cycles_bytes);
+size_t neogemm_bf16_profile_bytes(int64_t M, int64_t N, int variant);
+
 /* Text for a status code; replaces the std::cerr print at nemgemmV03.cu:387-390. Never NULL. */
 const char* neogemm_strerror(int status);
 
