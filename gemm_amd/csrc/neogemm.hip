@@ -5,7 +5,7 @@
 // round-to-nearest-even.  How it is computed shares nothing with it: the reference stages 64x64 tiles
 // with TMA and issues WGMMA from one warpgroup (v01.cu:215-237); here a workgroup of wave64s owns a
 // 256x256 (or smaller) macro-tile, stages 64-deep K slabs with direct-to-LDS buffer loads into a
-// double-buffered, XOR-swizzled LDS image, and feeds v_mfma_f32_32x32x16_bf16 from ds_read_b128 /
+// double-buffered, XOR-swizzled LDS image, and feeds v_mfma_f32_16x16x32_bf16 from ds_read_b128 /
 // ds_read_b64_tr_b16.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -37,24 +37,24 @@ static constexpr uint32_t OOB_OFFSET = 0x80000000u;  // >= every num_records thi
 //
 // K-major operand (rows of the matrix are K-contiguous: A[M,K], B[N,K]):
 //   image = ROWS x 64 B, row r at r*64, four 16-byte chunks per row; logical chunk c of row r lives
-//   at physical chunk c ^ swz_k(r).  An MFMA operand read has 32 lanes fetch the same logical chunk
-//   of 32 consecutive rows; swz_k makes any 8 consecutive rows cover the 8 slots of a 128-byte
-//   window and any 16 consecutive rows the 16 slots of a 256-byte window exactly once.
+//   at physical chunk c ^ swz_k(r).  An MFMA operand read (16 rows x 32 k) has 16 lanes fetch the
+//   same logical chunk of 16 consecutive rows; swz_k makes any 8 consecutive rows cover the 8 slots
+//   of a 128-byte window and any 16 consecutive rows the 16 slots of a 256-byte window exactly once.
 // MN-major operand (the K index is the slow one: B[K,N]):
 //   image = 32 x (ROWS*2) B, k-row at k*ROWS*2; logical chunk c (8 columns) of k-row k lives at
-//   physical chunk c ^ swz_mn(k & 3).  Read back with ds_read_b64_tr_b16: in each group of 16 lanes,
+//   physical chunk c ^ swz_mn(k).  Read back with ds_read_b64_tr_b16: in each group of 16 lanes,
 //   lanes 4r..4r+3 address k-row r (16 columns, 8 bytes per lane) and lane j receives the 4 k-values
-//   of column j.
+//   of column j.  A half-wave touches k-rows {0..3} and {8..11} (+4, +16), 32 bytes of each: swz_mn
+//   spreads those eight 32-byte pieces over the 64 banks.
 // Direct-to-LDS loads write 64 lanes x 16 B contiguously, so the swizzle is applied by choosing which
 // global chunk each lane fetches.
 // ---------------------------------------------------------------------------------------------
 __device__ __forceinline__ uint32_t swz_k(uint32_t row) {
   return (((row >> 2) & 1u) << 1) | (((row >> 1) ^ (row >> 3)) & 1u);
 }
-__device__ __forceinline__ uint32_t swz_mn(uint32_t k4) {
-  // k4 in 0..3 -> {0, 4, 10, 14}
-  uint32_t u = (k4 << 1) ^ (k4 >> 1);
-  return u << 1;
+__device__ __forceinline__ uint32_t swz_mn(uint32_t krow) {
+  // even values 0..14: (k & 3) picks the 32-byte pair, bit 3 of k the 128-byte half
+  return ((krow & 3u) << 1) | (((krow >> 3) & 1u) << 3);
 }
 
 // One 1 KiB direct-to-LDS load: lane i's 16 bytes at (rsrc.base + voff) land at lds + 16*i.
@@ -132,7 +132,7 @@ struct Operand {
 #pragma unroll
       for (int j = 0; j < IPW; ++j) {
         uint32_t krow = (wave * IPW + j) * KR + lane / CPR;
-        uint32_t c = (lane % CPR) ^ swz_mn(krow & 3);
+        uint32_t c = (lane % CPR) ^ swz_mn(krow);
         voff[j] = krow * (uint32_t)ld * 2 + c * 16;
         // A chunk that starts past the last column would wrap into the next k-row.
         if (r0 + (int)c * 8 >= rows_total) voff[j] = OOB_OFFSET;
@@ -170,36 +170,35 @@ struct Operand {
   __device__ __forceinline__ void advance() { base += kadv; }
 };
 
-// Per-lane constants for reading MFMA operand fragments (32 rows x 16 k per fragment) out of a slab image.
+// Per-lane constants for reading MFMA operand fragments out of a slab image.  A fragment is the
+// 16 rows x 32 k operand of v_mfma_f32_16x16x32_bf16: lane l holds row (l & 15), k = 8*(l >> 4) .. +7.
 template <int ROWS, bool KMAJOR, int NT>
 struct FragReader {
   static constexpr int ROWB = ROWS * 2;
   uint32_t lane_off[KMAJOR ? 1 : NT];
-  uint32_t xs[KMAJOR ? 2 : 1];
 
   __device__ __forceinline__ void init(int wrow0, int lane) {
     if constexpr (KMAJOR) {
-      lane_off[0] = (uint32_t)(wrow0 + (lane & 31)) * 64;
-#pragma unroll
-      for (int s = 0; s < 2; ++s) xs[s] = (((uint32_t)(2 * s + (lane >> 5))) ^ swz_k(lane & 15)) << 4;
+      const uint32_t row = lane & 15;
+      lane_off[0] = (uint32_t)(wrow0 + row) * 64 + ((((uint32_t)lane >> 4) ^ swz_k(row)) << 4);
     } else {
-      const uint32_t i = lane & 15, g1 = (lane >> 4) & 1, h = lane >> 5;
+      const uint32_t i = lane & 15, q = lane >> 4;
       const uint32_t tr_r = i >> 2, tr_c = i & 3;
+      const uint32_t krow = 8 * q + tr_r;  // the second read adds 4: same swizzle
 #pragma unroll
       for (int t = 0; t < NT; ++t) {
-        uint32_t chunk = (uint32_t)(wrow0 >> 3) + 4 * t + 2 * g1 + (tr_c >> 1);
-        lane_off[t] = (8 * h + tr_r) * ROWB + ((chunk ^ swz_mn(tr_r)) << 4) + ((tr_c & 1) << 3);
+        uint32_t chunk = (uint32_t)(wrow0 >> 3) + 2 * t + (tr_c >> 1);
+        lane_off[t] = krow * ROWB + ((chunk ^ swz_mn(krow)) << 4) + ((tr_c & 1) << 3);
       }
-      xs[0] = 0;
     }
   }
-  // fragment t (32 rows), k-step s (16 deep, 0 or 1) of the slab image at LDS address `img`
-  __device__ __forceinline__ bf16x8 read(uint32_t img, int t, int s) const {
+  // fragment t (16 rows, all 32 k) of the slab image at LDS address `img`
+  __device__ __forceinline__ bf16x8 read(uint32_t img, int t) const {
     if constexpr (KMAJOR) {
-      return lds_read_b128(img + lane_off[0] + t * 2048 + xs[s]);
+      return lds_read_b128(img + lane_off[0] + t * 1024);
     } else {
-      i16x4 lo = lds_read_tr16(img + lane_off[t] + (16 * s) * ROWB);
-      i16x4 hi = lds_read_tr16(img + lane_off[t] + (16 * s + 4) * ROWB);
+      i16x4 lo = lds_read_tr16(img + lane_off[t]);
+      i16x4 hi = lds_read_tr16(img + lane_off[t] + 4 * ROWB);
       i16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
       return __builtin_bit_cast(bf16x8, v);
     }
@@ -213,9 +212,9 @@ template <int BM, int BN, int WGM, int WGN, bool AK, bool BK, bool PROF = false>
 __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
   constexpr int NW = WGM * WGN;
   constexpr int WTM = BM / WGM, WTN = BN / WGN;
-  constexpr int TM = WTM / 32, TN = WTN / 32;
+  constexpr int TM = WTM / 16, TN = WTN / 16;
   constexpr uint32_t A_BYTES = BM * KT * 2, B_BYTES = BN * KT * 2, SLAB = A_BYTES + B_BYTES;
-  static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be a multiple of the 32x32 MFMA tile");
+  static_assert(WTM % 16 == 0 && WTN % 16 == 0, "wave tile must be a multiple of the 16x16 MFMA tile");
   using OpA = Operand<BM, AK, NW>;
   using OpB = Operand<BN, BK, NW>;
   constexpr int LA = OpA::IPW, LB = OpB::IPW, LPS = LA + LB;  // this wave's loads per slab
@@ -262,76 +261,72 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
   fa.init(wm * WTM, lane);
   fb.init(wn * WTN, lane);
 
-  f32x16 acc[TM][TN];
+  f32x4 acc[TM][TN];
 #pragma unroll
   for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int j = 0; j < TN; ++j)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+      for (int v = 0; v < 4; ++v) acc[i][j][v] = 0.f;
 
-  bf16x8 af[2][TM], bfr[2][TN];
+  static_assert(TM % 2 == 0, "the wave tile is processed in two halves of TM/2 fragment rows");
+  constexpr int HM = TM / 2;
+  bf16x8 af[TM], bfr[TN];  // one copy of each fragment; refreshed in place as soon as it is dead
 
-  // One k-step (16 deep): the MFMAs of fragment buffer `cur`, the LDS reads that fill the other
-  // buffer from slab image `img_next` / k-step `s_next`, and this wave's loads of one operand of a
-  // later slab into image `img_dma`.  The work is cut into groups — one direct-to-LDS load per group,
-  // the LDS reads in the first half of the groups — so that the wave never issues a burst of memory
-  // instructions: a burst backs up the vector-memory queue and the wave, which issues in order,
-  // cannot reach its next MFMA until the queue has drained.
-  auto kstep = [&](int cur, auto do_read, uint32_t img_next, int s_next, auto dma_a, auto dma_b, uint32_t img_dma) {
-    constexpr bool READ = decltype(do_read)::value;
-    constexpr bool DMA_A = decltype(dma_a)::value, DMA_B = decltype(dma_b)::value;
-    constexpr int NL = DMA_A ? LA : (DMA_B ? LB : 0);
-    constexpr int NG = NL > 0 ? (NL < TM * TN ? NL : TM * TN) : 2;   // groups
-    constexpr int MPG = (TM * TN) / NG;                              // MFMAs per group
-    static_assert((TM * TN) % NG == 0, "MFMAs must divide over the groups");
-    constexpr int RG = NG >= 2 ? NG / 2 : 1;                          // groups that carry LDS reads
-    constexpr int NFRAG = TM + TN;
-    constexpr int FPG = (NFRAG + RG - 1) / RG;                        // fragments read per group
+  auto img_of = [&](int slab) -> uint32_t { return lds0 + (uint32_t)(slab & (NSLAB - 1)) * SLAB; };
+
+  // Half a slab step: the MFMAs of fragment rows [HALF*HM, HALF*HM + HM) against every B fragment,
+  // column by column, with the LDS reads that refresh dead fragments and (DMA) this wave's loads of
+  // one operand of a later slab, one load after every few columns.  The wave issues in order, and
+  // whatever sits between two MFMAs beyond the 16 cycles the first one occupies the pipe is lost, so
+  // memory instructions are never issued in bursts.
+  //   HALF 0 reads the second-half A fragments of the slab being computed (image img_rd).
+  //   HALF 1 reads, from the next slab's image img_rd, the first-half A fragments and, after the last
+  //   MFMA that uses it, each B fragment.
+  auto half_step = [&](auto half, auto do_read, uint32_t img_rd, auto do_dma, uint32_t img_dma) {
+    constexpr int HALF = decltype(half)::value;
+    constexpr bool READ = decltype(do_read)::value, DMA = decltype(do_dma)::value;
+    constexpr int NL = DMA ? (HALF == 1 ? LA : LB) : 0;  // A part under half 1, B part under the next half 0
+    constexpr int APC = (HM + TN - 1) / TN;               // A fragments refreshed per column
     i32x4 rs;
-    if constexpr (DMA_A) rs = opa.rsrc();
-    if constexpr (DMA_B) rs = opb.rsrc();
-    static_for<NG>([&](auto gc) {
-      constexpr int g = decltype(gc)::value;
-      constexpr int f0 = g * FPG, f1 = (g + 1) * FPG < NFRAG ? (g + 1) * FPG : NFRAG;
-      constexpr bool READS = READ && g < RG && f0 < f1;
-      // LDS read instructions this group issues (an MN-major fragment takes two transposing reads)
-      constexpr int na = READS ? ((f1 < TM ? f1 : TM) - (f0 < TM ? f0 : TM)) : 0;
-      constexpr int nb = READS ? ((f1 - f0) - na) : 0;
-      constexpr int nread = na * (AK ? 1 : 2) + nb * (BK ? 1 : 2);
-      if constexpr (READS) {
+    if constexpr (DMA) rs = HALF == 1 ? opa.rsrc() : opb.rsrc();
+    static_for<TN>([&](auto cc) {
+      constexpr int c = decltype(cc)::value;
 #pragma unroll
-        for (int f = f0; f < f1; ++f) {
-          if (f < TM) af[cur ^ 1][f] = fa.read(img_next, f, s_next);
-          else bfr[cur ^ 1][f - TM] = fb.read(img_next + A_BYTES, f - TM, s_next);
-        }
-      }
-#pragma unroll
-      for (int m = g * MPG; m < (g + 1) * MPG; ++m) {
-        const int i = m / TN, j = m % TN;
+      for (int i = HALF * HM; i < HALF * HM + HM; ++i)
         // B fragment first: D rows index n, D columns index m, so a lane ends up with 4
         // consecutive n of one output row (an 8-byte store) instead of 4 rows of one column.
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[cur][j], af[cur][i], acc[i][j], 0, 0, 0);
+        acc[i][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bfr[c], af[i], acc[i][c], 0, 0, 0);
+      constexpr int a_lo = c * APC < HM ? c * APC : HM, a_hi = (c + 1) * APC < HM ? (c + 1) * APC : HM;
+      constexpr int nread = READ ? (a_hi - a_lo) * (AK ? 1 : 2) + (HALF == 1 ? (BK ? 1 : 2) : 0) : 0;
+      if constexpr (READ) {
+        if constexpr (HALF == 1) bfr[c] = fb.read(img_rd + A_BYTES, c);
+#pragma unroll
+        for (int f = a_lo; f < a_hi; ++f) {
+          if constexpr (HALF == 0) af[HM + f] = fa.read(img_rd, HM + f);
+          else af[f] = fa.read(img_rd, f);
+        }
       }
-      // within the group: one MFMA first, then the LDS reads, then the rest of the MFMAs
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, HM, 0);
       if constexpr (nread > 0) __builtin_amdgcn_sched_group_barrier(0x100, nread, 0);
-      if constexpr (MPG > 1) __builtin_amdgcn_sched_group_barrier(0x008, MPG - 1, 0);
-      if constexpr (NL > 0) {
+      // loads: NL of them spread over the TN columns
+      constexpr int l_lo = c * NL / TN, l_hi = (c + 1) * NL / TN;
+      if constexpr (l_hi > l_lo) {
         __builtin_amdgcn_sched_barrier(0);
-        if constexpr (DMA_A) {
-          if constexpr (g < LA) opa.issue_one(rs, img_dma, g);
-        } else {
-          if constexpr (g < LB) opb.issue_one(rs, img_dma + A_BYTES, g);
+#pragma unroll
+        for (int l = l_lo; l < l_hi; ++l) {
+          if constexpr (HALF == 1) opa.issue_one(rs, img_dma, l);
+          else opb.issue_one(rs, img_dma + A_BYTES, l);
         }
         __builtin_amdgcn_sched_barrier(0);
       }
     });
-    if constexpr (DMA_A) opa.advance();
-    if constexpr (DMA_B) opb.advance();
+    if constexpr (DMA) {
+      if constexpr (HALF == 1) opa.advance();
+      else opb.advance();
+    }
   };
 
-  auto img_of = [&](int slab) -> uint32_t { return lds0 + (uint32_t)(slab & (NSLAB - 1)) * SLAB; };
   auto load_slab_burst = [&](int j) {
     if (j == nslab - 1 && k_tail != KT) {
       opa.mask_k_tail(k_tail, wave, lane);
@@ -370,16 +365,22 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
   };
   using T = std::true_type;
   using F = std::false_type;
+  using H0 = std::integral_constant<int, 0>;
+  using H1 = std::integral_constant<int, 1>;
 
-  // Ring of NSLAB slab images; slab j lives in image j % NSLAB.  Steady state, for slab j:
-  //   k-step 0 of slab j    reads the fragments of k-step 1 of slab j
-  //   sync                  all waves are done reading slab j, slab j+1 has landed everywhere
-  //   k-step 1 of slab j    reads k-step 0 of slab j+1, streams the A part of slab j+4 into image j%4
-  //   k-step 0 of slab j+1  reads k-step 1 of slab j+1, streams the B part of slab j+4
-  // so a load has at least two slab-times to land and loads leave the wave one at a time.
+  // Ring of NSLAB slab images; slab j lives in image j % NSLAB.  The work on slab j is
+  //   half 0   MFMAs of the first-half rows; reads the second-half A fragments of slab j;
+  //            streams the B part of slab j+3 into image (j+3)%4
+  //   sync     every wave has all fragments of slab j in registers (image j%4 may be overwritten)
+  //            and slab j+1 has landed for all of them
+  //   half 1   MFMAs of the second-half rows; reads from slab j+1 the first-half A fragments and
+  //            each B fragment right after its last use; streams the A part of slab j+4 into image j%4
+  // so a load has at least two slab-times to land, loads leave the wave one at a time, and only one
+  // copy of each fragment is held in registers.  The loop below is rotated: one iteration is
+  // sync, half 1 of slab j, half 0 of slab j+1.
   {
     const int npre = nslab < NSLAB ? nslab : NSLAB;
-    for (int j = 0; j < npre; ++j) load_slab_burst(j);
+    for (int jj = 0; jj < npre; ++jj) load_slab_burst(jj);
     // slab 0 landed: everything but the later slabs' loads
     if (npre == 4) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * LPS) : "memory");
     else if (npre == 3) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * LPS) : "memory");
@@ -389,10 +390,10 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
     asm volatile("" ::: "memory");
   }
 #pragma unroll
-  for (int t = 0; t < TM; ++t) af[0][t] = fa.read(img_of(0), t, 0);
+  for (int t = 0; t < HM; ++t) af[t] = fa.read(img_of(0), t);
 #pragma unroll
-  for (int t = 0; t < TN; ++t) bfr[0][t] = fb.read(img_of(0) + A_BYTES, t, 0);
-  kstep(0, T{}, img_of(0), 1, F{}, F{}, 0);
+  for (int t = 0; t < TN; ++t) bfr[t] = fb.read(img_of(0) + A_BYTES, t);
+  half_step(H0{}, T{}, img_of(0), F{}, 0);
 
   int j = 0;
   // steady: slab j+4 exists and is not the last one (the last may need its K tail masked)
@@ -401,46 +402,44 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
     for (int u = 0; u < NSLAB; ++u) {
       const uint32_t img_free = lds0 + u * SLAB, img_next = lds0 + ((u + 1) & (NSLAB - 1)) * SLAB;
       sync(std::integral_constant<int, 2 * LPS>{});
-      kstep(1, T{}, img_next, 0, T{}, F{}, img_free);
-      kstep(0, T{}, img_next, 1, F{}, T{}, img_free);
+      half_step(H1{}, T{}, img_next, T{}, img_free);
+      half_step(H0{}, T{}, img_next, T{}, img_free);
     }
   }
   // tail: runtime slab indices, loads in a burst, conservative waits
   for (; j + 1 < nslab; ++j) {
     sync(std::integral_constant<int, 0>{});
     if (j + NSLAB < nslab) load_slab_burst(j + NSLAB);
-    kstep(1, T{}, img_of(j + 1), 0, F{}, F{}, 0);
-    kstep(0, T{}, img_of(j + 1), 1, F{}, F{}, 0);
+    half_step(H1{}, T{}, img_of(j + 1), F{}, 0);
+    half_step(H0{}, T{}, img_of(j + 1), F{}, 0);
   }
-  kstep(1, F{}, 0, 0, F{}, F{}, 0);
-  // every load was waited for by the last sync (or the prologue when there is one slab)
+  // second half of the last slab: its fragments are in registers or on their way from LDS; every
+  // load was waited for by the last sync (or the prologue when there is one slab)
+  half_step(H1{}, F{}, 0, F{}, 0);
 
   unsigned long long t_main = 0;
   if constexpr (PROF) t_main = __builtin_readcyclecounter();
 
-  // Epilogue: lane holds, per 32x32 tile, output row (lane & 31) and four runs of 4 consecutive columns.
-  const int row_l = lane & 31, colq = (lane >> 5) * 4;
+  // Epilogue: lane holds, per 16x16 tile, output row (lane & 15) and 4 consecutive columns 4*(lane >> 4)..+3.
+  const int row_l = lane & 15, colq = (lane >> 4) * 4;
   if (p.ksplit == 1) {
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
-      const int row = m0 + wm * WTM + i * 32 + row_l;
+      const int row = m0 + wm * WTM + i * 16 + row_l;
       if (row >= p.M) continue;
       char* crow = p.C + (size_t)row * p.ldc * 2;
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
+        const int col = n0 + wn * WTN + j * 16 + colq;
+        bf16x4 o;
 #pragma unroll
-        for (int b = 0; b < 4; ++b) {
-          const int col = n0 + wn * WTN + j * 32 + 8 * b + colq;
-          bf16x4 o;
+        for (int r = 0; r < 4; ++r) o[r] = (__bf16)acc[i][j][r];
+        if (col + 3 < p.N) {
+          *(bf16x4*)(crow + (size_t)col * 2) = o;
+        } else {
 #pragma unroll
-          for (int r = 0; r < 4; ++r) o[r] = (__bf16)acc[i][j][4 * b + r];
-          if (col + 3 < p.N) {
-            *(bf16x4*)(crow + (size_t)col * 2) = o;
-          } else {
-#pragma unroll
-            for (int r = 0; r < 4; ++r)
-              if (col + r < p.N) *(__bf16*)(crow + (size_t)(col + r) * 2) = o[r];
-          }
+          for (int r = 0; r < 4; ++r)
+            if (col + r < p.N) *(__bf16*)(crow + (size_t)(col + r) * 2) = o[r];
         }
       }
     }
@@ -449,22 +448,18 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
     const bool vec = (p.N & 3) == 0;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
-      const int row = m0 + wm * WTM + i * 32 + row_l;
+      const int row = m0 + wm * WTM + i * 16 + row_l;
       if (row >= p.M) continue;
       float* wrow = wsz + (size_t)row * p.N;
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
+        const int col = n0 + wn * WTN + j * 16 + colq;
+        if (vec && col + 3 < p.N) {
+          *(f32x4*)(wrow + col) = acc[i][j];
+        } else {
 #pragma unroll
-        for (int b = 0; b < 4; ++b) {
-          const int col = n0 + wn * WTN + j * 32 + 8 * b + colq;
-          if (vec && col + 3 < p.N) {
-            f32x4 o = {acc[i][j][4 * b], acc[i][j][4 * b + 1], acc[i][j][4 * b + 2], acc[i][j][4 * b + 3]};
-            *(f32x4*)(wrow + col) = o;
-          } else {
-#pragma unroll
-            for (int r = 0; r < 4; ++r)
-              if (col + r < p.N) wrow[col + r] = acc[i][j][4 * b + r];
-          }
+          for (int r = 0; r < 4; ++r)
+            if (col + r < p.N) wrow[col + r] = acc[i][j][r];
         }
       }
     }
