@@ -57,15 +57,30 @@ __device__ __forceinline__ uint32_t swz_mn(uint32_t krow) {
   return ((krow & 3u) << 1) | (((krow >> 3) & 1u) << 3);
 }
 
-// One 1 KiB direct-to-LDS load: lane i's 16 bytes at (rsrc.base + voff) land at lds + 16*i.
-// The compiler is not told that this touches LDS; ordering against ds_read is done by hand with
+// Direct-to-LDS loads.  One instruction moves 1 KiB: lane i's 16 bytes at (rsrc.base + voff + OFF)
+// land at LDS address M0 + OFF + 16*i.  M0 is written once per run of loads (a scalar write, a wait
+// state, then up to four loads told apart by the 12-bit instruction offset, which moves the global
+// and the LDS address alike — the per-lane offsets are built with that in mind): a load then costs
+// the wave one issue slot, which fits behind a 16-cycle MFMA, where m0-write + nop + load does not.
+// The compiler is not told that these touch LDS; ordering against ds_read is done by hand with
 // s_waitcnt vmcnt + s_barrier (a builtin load would make the compiler wait vmcnt(0) before every
 // LDS read and serialise the pipeline).
-__device__ __forceinline__ void dma16(i32x4 rsrc, uint32_t lds, uint32_t voff) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
-               :
-               : "s"(lds), "v"(voff), "s"(rsrc)
-               : "memory");
+__device__ __forceinline__ void dma_set_m0(uint32_t lds) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0" : : "s"(lds) : "memory");
+}
+template <int OFF>
+__device__ __forceinline__ void dma16(i32x4 rsrc, uint32_t voff) {
+  static_assert(OFF >= 0 && OFF < 4096, "12-bit instruction offset");
+  asm volatile("buffer_load_dwordx4 %0, %1, 0 offen offset:%2 lds" : : "v"(voff), "s"(rsrc), "n"(OFF) : "memory");
+}
+
+// acc += A(16x32) * B(32x16) with the accumulator pinned in AGPRs and written in place.  Written as
+// asm because the builtin lets the register allocator pick a destination different from the source
+// accumulator; with all 256 AGPRs holding accumulators that ends in a storm of v_accvgpr copies at
+// the loop back-edge.  Being opaque to the compiler, no hazard NOPs are inserted for it: the caller
+// keeps reads of an accumulator away from the MFMA that wrote it (see the s_nop before the epilogue).
+__device__ __forceinline__ void mfma_16x16x32(f32x4& acc, bf16x8 a, bf16x8 b) {
+  asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
 }
 
 __device__ __forceinline__ bf16x8 lds_read_b128(uint32_t addr) {
@@ -105,67 +120,75 @@ struct Operand {
   static constexpr int ROWB = ROWS * 2;     // bytes per k-row of an MN-major image
   static constexpr int CPR = ROWS / 8;      // 16-byte chunks per k-row (MN-major)
   static constexpr int KR = 64 / CPR;       // k-rows per wave-load (MN-major)
-  static_assert(NINSTR % NW == 0 && IPW >= 1, "slab loads must divide evenly over the waves");
+  static_assert(NINSTR % NW == 0 && IPW >= 1 && IPW <= 4, "slab loads must divide evenly over the waves, at most 4 each");
   static_assert(KMAJOR || ROWS >= 128, "MN-major swizzle needs >= 16 chunks per k-row");
 
   uint32_t voff[IPW];
-  uint64_t base, end;
+  uint64_t base;
   uint32_t kadv;
   uint32_t lds_w;
 
-  __device__ __forceinline__ void init(const char* ptr, long ld, int rows_total, int r0, int k_begin, int K,
-                                       int wave, int lane) {
+  // Every lane offset that would leave the matrix is replaced by OOB_OFFSET, which the buffer range
+  // check (num_records = 2 GiB, constant) turns into a zero fill without a memory access; all other
+  // offsets address bytes inside the matrix, so the resource needs no exact size and only its base
+  // moves along K.
+  __device__ __forceinline__ void init(const char* ptr, long ld, int rows_total, int r0, int k_begin, int wave,
+                                       int lane) {
     if constexpr (KMAJOR) {
       base = (uint64_t)ptr + ((uint64_t)r0 * ld + k_begin) * 2;
-      end = (uint64_t)ptr + ((uint64_t)(rows_total - 1) * ld + K) * 2;
       kadv = KT * 2;
 #pragma unroll
       for (int j = 0; j < IPW; ++j) {
         uint32_t row = (wave * IPW + j) * 16 + (lane >> 2);
         uint32_t c = (lane & 3) ^ swz_k(row);
-        voff[j] = row * (uint32_t)ld * 2 + c * 16;
+        // load j carries instruction offset j*1024 (see dma16); row >= 16*j and ld >= 32 keep this >= 0
+        voff[j] = row * (uint32_t)ld * 2 + c * 16 - j * 1024;
+        if (r0 + (int)row >= rows_total) voff[j] = OOB_OFFSET;
       }
     } else {
       base = (uint64_t)ptr + ((uint64_t)k_begin * ld + r0) * 2;
-      end = (uint64_t)ptr + ((uint64_t)(K - 1) * ld + rows_total) * 2;
       kadv = KT * (uint32_t)ld * 2;
 #pragma unroll
       for (int j = 0; j < IPW; ++j) {
         uint32_t krow = (wave * IPW + j) * KR + lane / CPR;
         uint32_t c = (lane % CPR) ^ swz_mn(krow);
-        voff[j] = krow * (uint32_t)ld * 2 + c * 16;
-        // A chunk that starts past the last column would wrap into the next k-row.
+        // krow >= KR*j and ld >= ROWS keep this >= 0
+        voff[j] = krow * (uint32_t)ld * 2 + c * 16 - j * 1024;
+        // a chunk past the last column would wrap into the next k-row (rows_total % 8 == 0: no straddling)
         if (r0 + (int)c * 8 >= rows_total) voff[j] = OOB_OFFSET;
       }
     }
     lds_w = wave * IPW * 1024;
   }
 
-  // K-major only: drop the chunks of the last, partial slab (they would wrap into the next row).
-  // An MN-major slab needs nothing: its k-rows past K lie beyond the end of the buffer.
+  // Last, partial slab of depth krem: drop what lies past K (K-major: chunks that would wrap into the
+  // next row; MN-major: whole k-rows).
   __device__ __forceinline__ void mask_k_tail(int krem, int wave, int lane) {
-    if constexpr (KMAJOR) {
 #pragma unroll
-      for (int j = 0; j < IPW; ++j) {
+    for (int j = 0; j < IPW; ++j) {
+      if constexpr (KMAJOR) {
         uint32_t row = (wave * IPW + j) * 16 + (lane >> 2);
         uint32_t c = (lane & 3) ^ swz_k(row);
         if ((int)c * 8 >= krem) voff[j] = OOB_OFFSET;
+      } else {
+        uint32_t krow = (wave * IPW + j) * KR + lane / CPR;
+        if ((int)krow >= krem) voff[j] = OOB_OFFSET;
       }
     }
   }
 
   __device__ __forceinline__ i32x4 rsrc() const {
-    const uint64_t rem = end - base;
-    const uint32_t nr = (rem >> 31) ? 0x80000000u : (uint32_t)rem;
     i32x4 r;
     r[0] = (int)(uint32_t)base;
-    r[1] = (int)((uint32_t)(base >> 32) & 0xffffu);
-    r[2] = (int)nr;
+    r[1] = (int)(uint32_t)(base >> 32);  // a 48-bit address: bits 16.. (stride, swizzle) stay 0
+    r[2] = (int)0x80000000u;
     r[3] = 0x00020000;
     return r;
   }
-  __device__ __forceinline__ void issue_one(i32x4 r, uint32_t lds_img, int j) const {
-    dma16(r, lds_img + lds_w + j * 1024, voff[j]);
+  // load j of this wave for the slab image at lds_img; M0 must hold lds_img + lds_w (dma_set_m0)
+  template <int J>
+  __device__ __forceinline__ void issue_one(i32x4 r) const {
+    dma16<J * 1024>(r, voff[J]);
   }
   __device__ __forceinline__ void advance() { base += kadv; }
 };
@@ -254,8 +277,8 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
 
   OpA opa;
   OpB opb;
-  opa.init(p.A, p.lda, p.M, m0, k_begin, p.K, wave, lane);
-  opb.init(p.B, p.ldb, p.N, n0, k_begin, p.K, wave, lane);
+  opa.init(p.A, p.lda, p.M, m0, k_begin, wave, lane);
+  opb.init(p.B, p.ldb, p.N, n0, k_begin, wave, lane);
   FragReader<BM, AK, TM> fa;
   FragReader<BN, BK, TN> fb;
   fa.init(wm * WTM, lane);
@@ -289,14 +312,17 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
     constexpr int NL = DMA ? (HALF == 1 ? LA : LB) : 0;  // A part under half 1, B part under the next half 0
     constexpr int APC = (HM + TN - 1) / TN;               // A fragments refreshed per column
     i32x4 rs;
-    if constexpr (DMA) rs = HALF == 1 ? opa.rsrc() : opb.rsrc();
+    if constexpr (DMA) {
+      rs = HALF == 1 ? opa.rsrc() : opb.rsrc();
+      dma_set_m0(HALF == 1 ? img_dma + opa.lds_w : img_dma + A_BYTES + opb.lds_w);
+    }
     static_for<TN>([&](auto cc) {
       constexpr int c = decltype(cc)::value;
 #pragma unroll
       for (int i = HALF * HM; i < HALF * HM + HM; ++i)
         // B fragment first: D rows index n, D columns index m, so a lane ends up with 4
         // consecutive n of one output row (an 8-byte store) instead of 4 rows of one column.
-        acc[i][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bfr[c], af[i], acc[i][c], 0, 0, 0);
+        mfma_16x16x32(acc[i][c], bfr[c], af[i]);
       constexpr int a_lo = c * APC < HM ? c * APC : HM, a_hi = (c + 1) * APC < HM ? (c + 1) * APC : HM;
       constexpr int nread = READ ? (a_hi - a_lo) * (AK ? 1 : 2) + (HALF == 1 ? (BK ? 1 : 2) : 0) : 0;
       if constexpr (READ) {
@@ -307,18 +333,15 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
           else af[f] = fa.read(img_rd, f);
         }
       }
-      __builtin_amdgcn_sched_group_barrier(0x008, HM, 0);
-      if constexpr (nread > 0) __builtin_amdgcn_sched_group_barrier(0x100, nread, 0);
+      (void)nread;
       // loads: NL of them spread over the TN columns
       constexpr int l_lo = c * NL / TN, l_hi = (c + 1) * NL / TN;
       if constexpr (l_hi > l_lo) {
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int l = l_lo; l < l_hi; ++l) {
-          if constexpr (HALF == 1) opa.issue_one(rs, img_dma, l);
-          else opb.issue_one(rs, img_dma + A_BYTES, l);
-        }
-        __builtin_amdgcn_sched_barrier(0);
+        static_for<l_hi - l_lo>([&](auto lc) {
+          constexpr int l = l_lo + decltype(lc)::value;
+          if constexpr (HALF == 1) opa.template issue_one<l>(rs);
+          else opb.template issue_one<l>(rs);
+        });
       }
     });
     if constexpr (DMA) {
@@ -333,10 +356,10 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
       opb.mask_k_tail(k_tail, wave, lane);
     }
     const i32x4 ra = opa.rsrc(), rb = opb.rsrc();
-#pragma unroll
-    for (int i = 0; i < LA; ++i) opa.issue_one(ra, img_of(j), i);
-#pragma unroll
-    for (int i = 0; i < LB; ++i) opb.issue_one(rb, img_of(j) + A_BYTES, i);
+    dma_set_m0(img_of(j) + opa.lds_w);
+    static_for<LA>([&](auto lc) { opa.template issue_one<decltype(lc)::value>(ra); });
+    dma_set_m0(img_of(j) + A_BYTES + opb.lds_w);
+    static_for<LB>([&](auto lc) { opb.template issue_one<decltype(lc)::value>(rb); });
     opa.advance();
     opb.advance();
   };
@@ -417,6 +440,14 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
   // load was waited for by the last sync (or the prologue when there is one slab)
   half_step(H1{}, F{}, 0, F{}, 0);
 
+  // The last MFMAs must have left the pipe before their accumulators are read, and the compiler,
+  // which sees neither MFMAs nor hazard here, inserts nothing.  Volatile asm statements keep their
+  // order, so the empty ones below, which redefine every accumulator, pin all later reads behind the NOPs.
+  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int jn = 0; jn < TN; ++jn) asm volatile("" : "+a"(acc[i][jn]));
   unsigned long long t_main = 0;
   if constexpr (PROF) t_main = __builtin_readcyclecounter();
 
@@ -658,7 +689,17 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
   a.ldc = ldc;
   a.K = (int)K;
   const VariantInfo& vi = kVariants[v];
-  if ((!ak && vi.bm < 128) || (!bk && vi.bn < 128)) return NEOGEMM_ERR_UNSUPPORTED;
+  // What the tile kernels assume about an operand (see Operand::init): an MN-major tile needs >= 128
+  // rows for its swizzle, ld >= tile rows and a row count that is a multiple of 8 (16-byte chunks must
+  // not straddle the matrix edge), a K-major one ld >= 32, so that the per-lane offsets, which are
+  // biased by the instruction offsets of the loads, stay non-negative.
+  const bool fits = (ak ? a.lda >= 32 : (vi.bm >= 128 && a.lda >= vi.bm && (a.M & 7) == 0)) &&
+                    (bk ? a.ldb >= 32 : (vi.bn >= 128 && a.ldb >= vi.bn && (a.N & 7) == 0));
+  if (!fits) {
+    if (variant != NEOGEMM_VARIANT_AUTO) return NEOGEMM_ERR_UNSUPPORTED;
+    return run(A, B, C, M, N, K, lda, ldb, ldc, b_layout, c_layout, workspace, workspace_bytes, hip_stream,
+               NEOGEMM_VARIANT_GENERIC, 1, 0, nullptr);
+  }
   a.ntm = ceil_div(a.M, vi.bm);
   a.ntn = ceil_div(a.N, vi.bn);
   if ((int64_t)a.ntm * a.ntn > 0x7fffffff) return NEOGEMM_ERR_UNSUPPORTED;
