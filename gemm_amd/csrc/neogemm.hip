@@ -614,7 +614,9 @@ static void plan(int64_t M, int64_t N, int64_t K, bool aligned, int* variant, in
     *split_k = 1;
     return;
   }
-  int v = NEOGEMM_VARIANT_T256x256_W8;
+  // One wave per SIMD with a 128x128 wave tile reads the least LDS per flop; below ~64 such tiles the
+  // 128x128 macro-tile (4 per CU's worth of work) fills the chip better.
+  int v = NEOGEMM_VARIANT_T256x256_W4;
   if (M <= 128 || N <= 128 || (int64_t)ceil_div(M, 256) * ceil_div(N, 256) < 64) v = NEOGEMM_VARIANT_T128x128_W4;
   const int64_t tiles = (int64_t)ceil_div(M, kVariants[v].bm) * ceil_div(N, kVariants[v].bn);
   const int64_t ktiles = ceil_div(K, KT);

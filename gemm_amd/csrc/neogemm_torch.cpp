@@ -12,8 +12,8 @@
 //  * the launch goes to torch's current stream, not the legacy default stream (nemgemmV03.cu:383);
 //  * no state is cached between calls (the reference caches TMA descriptors keyed on shape only,
 //    nemgemmV03.cu:27-30,359-371, which goes stale when another tensor of the same shape is passed).
-#include <c10/hip/HIPGuard.h>
-#include <c10/hip/HIPStream.h>
+#include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 #include <torch/extension.h>
 
 #include <string>
@@ -49,11 +49,12 @@ torch::Tensor& workspace_for(const torch::Tensor& like, size_t bytes) {
 
 void run(const torch::Tensor& A, const torch::Tensor& B, torch::Tensor& C, int64_t M, int64_t N, int64_t K,
          int64_t lda, int64_t ldb, int64_t ldc, int b_layout, int c_layout) {
-  c10::hip::HIPGuard guard(A.device());
+  // PyTorch-ROCm names its HIP devices "cuda"; these are the guard and stream accessors for that naming
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(A.device());
   const size_t need = neogemm_bf16_workspace_bytes(M, N, K);
   void* ws = nullptr;
   if (need) ws = workspace_for(A, need).data_ptr();
-  hipStream_t stream = c10::hip::getCurrentHIPStream(A.get_device()).stream();
+  hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(A.get_device()).stream();
   const int st = neogemm_bf16(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, lda, ldb, ldc, b_layout, c_layout,
                               ws, need, (void*)stream);
   TORCH_CHECK(st == NEOGEMM_OK, "neogemm_bf16 failed: ", neogemm_strerror(st));

@@ -1,0 +1,97 @@
+"""The C ABI of include/neogemm.h without a GPU: the library loads, exports every declared symbol, and
+its host-only entry points (plan, workspace size, error text, argument validation that returns before any
+HIP call) behave as documented.  No kernel is launched here."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from gemm_amd import _abi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "neogemm.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(neogemm_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_entry_points():
+    names = declared_functions()
+    for must in ("neogemm_bf16", "neogemm_bf16_workspace_bytes", "neogemm_bf16_variant", "neogemm_bf16_plan",
+                 "neogemm_bf16_profile", "neogemm_bf16_profile_bytes", "neogemm_strerror", "neogemm_version"):
+        assert must in names
+
+
+def test_library_exports_every_declared_symbol():
+    lib = ctypes.CDLL(_abi.LIB_PATH)
+    for name in declared_functions():
+        assert hasattr(lib, name), f"{name} is declared in include/neogemm.h but not exported"
+    # and the ctypes prototypes cover exactly the header
+    assert sorted(_abi.PROTOTYPES) == declared_functions()
+
+
+def test_header_cites_the_reference_for_each_entry_point():
+    text = open(HEADER).read()
+    for cite in ("nemgemmV03.cu:343-391", "v01.cu:189-270", "v01.cu:254-262", "nemgemmV03.cu:387-390",
+                 "v01.cu:304-311", "cublass/matmul.cu:99-106"):
+        assert cite in text
+
+
+def test_version_and_strerror():
+    assert "gfx950" in _abi.version()
+    assert _abi.strerror(0) == "success"
+    for st in (_abi.ERR_BAD_ARG, _abi.ERR_WORKSPACE, _abi.ERR_UNSUPPORTED, _abi.ERR_LAUNCH, -99):
+        s = _abi.strerror(st)
+        assert isinstance(s, str) and s and s != "success"
+
+
+def test_plan_for_the_benchmark_configs():
+    # square compute-bound shapes run a 256x256 tile kernel without split-K
+    for n in (4096, 8192):
+        v, s = _abi.plan(n, n, n)
+        assert v in (_abi.VARIANT_T256x256_W4, _abi.VARIANT_T256x256_W8) and s == 1
+    # shapes with few output tiles split K and need a workspace of split * M * N floats
+    for M, N, K in ((16, 14336, 4096), (64, 14336, 4096), (128, 14336, 4096), (1024, 1024, 32768), (512, 512, 512)):
+        v, s = _abi.plan(M, N, K)
+        assert v != _abi.VARIANT_GENERIC and s >= 1
+        assert _abi.workspace_bytes(M, N, K) == (s * M * N * 4 if s > 1 else 0)
+    assert _abi.plan(1024, 1024, 32768)[1] > 1
+    # unaligned problems go to the generic kernel
+    assert _abi.plan(100, 100, 100, aligned=False) == (_abi.VARIANT_GENERIC, 1)
+    assert _abi.workspace_bytes(0, 5, 5) == 0 and _abi.workspace_bytes(5, 5, 0) == 0
+
+
+def test_argument_validation_returns_before_touching_the_gpu():
+    bad = _abi.ERR_BAD_ARG
+    p = 0x1000  # never dereferenced: every call below is rejected, or is a no-op, on the host
+    assert _abi.gemm_raw(p, p, p, -1, 4, 4, 4, 4, 4, 0, 0) == bad
+    assert _abi.gemm_raw(p, p, p, 4, 4, 4, 4, 4, 4, 2, 0) == bad        # unknown b_layout
+    assert _abi.gemm_raw(p, p, p, 4, 4, 4, 4, 4, 4, 0, 7) == bad        # unknown c_layout
+    assert _abi.gemm_raw(p, p, p, 4, 4, 4, 3, 4, 4, 0, 0) == bad        # lda < K
+    assert _abi.gemm_raw(p, p, p, 4, 4, 4, 4, 3, 4, 0, 0) == bad        # ldb < N for [K,N]
+    assert _abi.gemm_raw(p, p, p, 4, 8, 4, 4, 3, 8, 1, 0) == bad        # ldb < K for [N,K]
+    assert _abi.gemm_raw(p, p, p, 4, 4, 4, 4, 4, 3, 0, 0) == bad        # ldc < N row-major
+    assert _abi.gemm_raw(p, p, p, 8, 4, 4, 4, 4, 4, 0, 1) == bad        # ldc < M column-major
+    assert _abi.gemm_raw(0, p, p, 4, 4, 4, 4, 4, 4, 0, 0) == bad        # null A
+    assert _abi.gemm_raw(p, p, 0, 4, 4, 4, 4, 4, 4, 0, 0) == bad        # null C
+    assert _abi.gemm_raw(p, p, p, 4, 4, 4, 4, 4, 4, 0, 0, variant=99) == bad
+    assert _abi.gemm_raw(p, p, p, 4, 4, 4, 4, 4, 4, 0, 0, variant=0, split_k=-1) == bad
+    # empty problems are no-ops
+    assert _abi.gemm_raw(0, 0, 0, 0, 4, 4, 4, 4, 4, 0, 0) == _abi.OK
+    assert _abi.gemm_raw(0, 0, 0, 4, 0, 4, 4, 4, 4, 0, 0) == _abi.OK
+
+
+def test_plan_rejects_null_outputs():
+    lib = _abi.load()
+    assert lib.neogemm_bf16_plan(4, 4, 4, 0, 0, 1, None, None) == _abi.ERR_BAD_ARG
+
+
+def test_profile_bytes():
+    lib = _abi.load()
+    assert lib.neogemm_bf16_profile_bytes(8192, 8192, _abi.VARIANT_T256x256_W8) == 1024 * 8 * 4 * 8
+    assert lib.neogemm_bf16_profile_bytes(8192, 8192, _abi.VARIANT_T256x256_W4) == 1024 * 4 * 4 * 8
+    assert lib.neogemm_bf16_profile_bytes(0, 8, _abi.VARIANT_T256x256_W4) == 0

@@ -1,0 +1,385 @@
+"""GPU parity tests: the HIP path, called through the C ABI (gemm_amd -> ctypes -> libneogemm.so) and
+through the built neoGEMM module, against the CPU oracle on the same seeded inputs.
+
+Tolerance (stated by the task): <= 1 bf16 ulp per element and <= 1e-3 relative Frobenius error against
+the fp32-accumulated CPU product rounded to bf16 — see oracle.gemm_oracle.assert_parity for how elements
+that cancel to nearly zero are treated.  Known-answer cases (identity, one-hot, ones, small integers) do
+not depend on summation order and are compared bit for bit.
+
+The reference can only run M, N, K that are multiples of 64 (nemgemmV03.cu:375) and has no tests; ragged,
+skinny and unaligned shapes are this build's own ground and are pinned by the oracle alone.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import gemm_amd as g
+from gemm_amd import _abi
+from oracle import gemm_oracle as o
+
+pytestmark = pytest.mark.gpu
+
+TILE_VARIANTS = [g.VARIANT_T256x256_W8, g.VARIANT_T256x256_W4, g.VARIANT_T128x128_W4, g.VARIANT_T256x128_W8,
+                 g.VARIANT_T128x256_W8]
+ALL_VARIANTS = [g.VARIANT_GENERIC] + TILE_VARIANTS
+
+
+def run_abi(A, B, dev, b_layout=g.B_KN, c_layout=g.C_ROW, variant=None, split_k=0, group_m=0):
+    """A [M,K] and B ([K,N] or [N,K]) are CPU bf16 tensors; returns the [M,N] result on the CPU."""
+    M, K = A.shape
+    N = B.shape[1] if b_layout == g.B_KN else B.shape[0]
+    Ad, Bd = A.to(dev), B.to(dev)
+    shape = (M, N) if c_layout == g.C_ROW else (N, M)
+    C = torch.full(shape, float("nan"), dtype=torch.bfloat16, device=dev)   # poison: every element must be written
+    g.gemm_into(Ad, Bd, C, M, N, K, max(K, 1), max(N if b_layout == g.B_KN else K, 1),
+                max(N if c_layout == g.C_ROW else M, 1), b_layout, c_layout, variant, split_k, group_m)
+    torch.cuda.synchronize()
+    C = C.cpu()
+    return C if c_layout == g.C_ROW else C.t().contiguous()
+
+
+def layouts(Bkn, b_layout):
+    return Bkn if b_layout == g.B_KN else Bkn.t().contiguous()
+
+
+# ------------------------------------------------------------------------------------------------
+# known answers: bit-exact, every variant, every layout
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("variant", ALL_VARIANTS)
+@pytest.mark.parametrize("b_layout", [g.B_KN, g.B_NK])
+@pytest.mark.parametrize("c_layout", [g.C_ROW, g.C_COL])
+def test_identity_and_permutation(dev, variant, b_layout, c_layout):
+    n = 384
+    A, _ = o.make_inputs(n, n, n, seed=1)
+    I = torch.eye(n, dtype=torch.bfloat16)
+    assert torch.equal(run_abi(A, layouts(I, b_layout), dev, b_layout, c_layout, variant), A)
+    perm = torch.randperm(n, generator=torch.Generator().manual_seed(2))
+    P = torch.zeros(n, n, dtype=torch.bfloat16)
+    P[torch.arange(n), perm] = 1
+    assert torch.equal(run_abi(P, layouts(A, b_layout), dev, b_layout, c_layout, variant), A[perm])
+
+
+@pytest.mark.parametrize("variant", ALL_VARIANTS)
+def test_exact_small_integers(dev, variant):
+    rng = np.random.default_rng(11)
+    M, N, K = 264, 328, 200   # ragged in M and N, partial last K slab
+    A = torch.from_numpy(rng.integers(-8, 9, size=(M, K)).astype(np.float32)).to(torch.bfloat16)
+    B = torch.from_numpy(rng.integers(-8, 9, size=(K, N)).astype(np.float32)).to(torch.bfloat16)
+    want = (A.to(torch.int64) @ B.to(torch.int64)).float().to(torch.bfloat16)   # |sum| < 2^24: fp32 exact
+    for b_layout in (g.B_KN, g.B_NK):
+        got = run_abi(A, layouts(B, b_layout), dev, b_layout, g.C_ROW, variant)
+        assert torch.equal(got, want)
+    if variant != g.VARIANT_GENERIC:
+        for split in (2, 3, 7):
+            assert torch.equal(run_abi(A, B, dev, variant=variant, split_k=split), want)
+
+
+@pytest.mark.parametrize("K", [8, 256, 264, 1000, 4096])
+def test_ones(dev, K):
+    A = torch.ones(40, K, dtype=torch.bfloat16)
+    B = torch.ones(K, 264, dtype=torch.bfloat16)
+    want = torch.tensor(float(K)).to(torch.bfloat16)   # 264 -> 264, 1000 -> 1000, exact sums then RNE
+    for variant in (None, g.VARIANT_T128x128_W4, g.VARIANT_T256x256_W4):
+        if variant is not None and K < 32:
+            continue   # the tile kernels need ld >= 32; the library's own choice covers such shapes
+        assert torch.all(run_abi(A, B, dev, variant=variant) == want)
+
+
+def test_rounding_is_nearest_even(dev):
+    # sums 257 and 259 sit exactly between two bf16 values: ties go to even (256, 260)
+    A = torch.ones(16, 264, dtype=torch.bfloat16)
+    for total, want in ((257, 256.0), (259, 260.0), (258, 258.0)):
+        B = torch.zeros(264, 16, dtype=torch.bfloat16)
+        B[:total] = 1
+        C = run_abi(A, B, dev)
+        assert torch.all(C.float() == want), (total, C[0, 0])
+
+
+# ------------------------------------------------------------------------------------------------
+# golden fixtures
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("name", ["tile64", "ragged", "odd", "skinny16", "tallk"])
+def test_golden(dev, name):
+    import os
+    z = np.load(os.path.join(os.path.dirname(__file__), "golden", f"{name}.npz"), allow_pickle=False)
+    A, B = o.from_bits(z["A"]), o.from_bits(z["B"])
+    want = o.from_bits(z["C_torch"])
+    for b_layout in (g.B_KN, g.B_NK):
+        for c_layout in (g.C_ROW, g.C_COL):
+            got = run_abi(A, layouts(B, b_layout), dev, b_layout, c_layout)
+            o.assert_parity(got, A, B, ref=want, what=f"{name} b{b_layout} c{c_layout}")
+
+
+# ------------------------------------------------------------------------------------------------
+# seeded random parity at the benchmark configurations
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("variant", [None] + ALL_VARIANTS)
+@pytest.mark.parametrize("b_layout", [g.B_KN, g.B_NK])
+@pytest.mark.parametrize("c_layout", [g.C_ROW, g.C_COL])
+def test_parity_512(dev, variant, b_layout, c_layout):
+    A, Bkn = o.make_inputs(512, 512, 512, seed=0)
+    got = run_abi(A, layouts(Bkn, b_layout), dev, b_layout, c_layout, variant)
+    o.assert_parity(got, A, Bkn, what=f"512^3 v{variant} b{b_layout} c{c_layout}")
+
+
+def check_big(dev, M, N, K, seed, b_layout=g.B_KN, variant=None, split_k=0, nrows=256):
+    """Full-size run; ulp and Frobenius against the full fp32 CPU product, the fp64-based bound on a
+    sample of rows (all rows when the problem is small)."""
+    A, Bkn = o.make_inputs(M, N, K, seed=seed)
+    got = run_abi(A, layouts(Bkn, b_layout), dev, b_layout, g.C_ROW, variant, split_k)
+    ref = o.ref_gemm(A, Bkn)
+    ulp = o.ulp_distance(o.bits_of(got), o.bits_of(ref))
+    assert bool(torch.isfinite(got.float()).all())
+    assert (ulp > 1).mean() <= 2e-3, f"{(ulp > 1).mean():.2e} of elements more than 1 raw ulp off"
+    rel = float(torch.linalg.norm(got.float() - ref.float()) / torch.linalg.norm(ref.float()))
+    assert rel <= o.TOL_REL_FRO, rel
+    idx = torch.arange(M) if M <= nrows else torch.cat([
+        torch.tensor([0, M - 1]), torch.randperm(M, generator=torch.Generator().manual_seed(seed))[:nrows - 2]])
+    return o.assert_parity(got[idx], A[idx], Bkn, ref=ref[idx], what=f"{M}x{N}x{K}")
+
+
+@pytest.mark.parametrize("b_layout", [g.B_KN, g.B_NK])
+def test_parity_4096(dev, b_layout):
+    check_big(dev, 4096, 4096, 4096, seed=1, b_layout=b_layout)
+
+
+def test_parity_8192_headline(dev):
+    check_big(dev, 8192, 8192, 8192, seed=2)
+
+
+@pytest.mark.parametrize("M", [16, 64, 128])
+@pytest.mark.parametrize("b_layout", [g.B_KN, g.B_NK])
+def test_parity_skinny(dev, M, b_layout):
+    check_big(dev, M, 14336, 4096, seed=3 + M, b_layout=b_layout)
+
+
+@pytest.mark.parametrize("b_layout", [g.B_KN, g.B_NK])
+def test_parity_irregular(dev, b_layout):
+    check_big(dev, 3000, 5120, 3584, seed=5, b_layout=b_layout)
+
+
+def test_parity_tall_k(dev):
+    r = check_big(dev, 1024, 1024, 32768, seed=6)
+    assert g.plan(1024, 1024, 32768)[1] > 1   # this shape runs split-K
+
+
+@pytest.mark.parametrize("variant", TILE_VARIANTS)
+@pytest.mark.parametrize("split", [2, 5, 16])
+def test_split_k(dev, variant, split):
+    M, N, K = 200, 392, 2056
+    A, Bkn = o.make_inputs(M, N, K, seed=8)
+    got = run_abi(A, Bkn, dev, variant=variant, split_k=split)
+    o.assert_parity(got, A, Bkn, what=f"split {split} v{variant}")
+
+
+# ------------------------------------------------------------------------------------------------
+# edges the reference never ran (it needs multiples of 64)
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("M,N,K", [(1, 1, 1), (1, 17, 5), (3, 1, 64), (7, 9, 8), (64, 64, 8), (65, 129, 72),
+                                   (255, 257, 24), (300, 520, 200), (16, 8, 4096), (129, 40, 520), (40, 1000, 31)])
+@pytest.mark.parametrize("b_layout", [g.B_KN, g.B_NK])
+@pytest.mark.parametrize("c_layout", [g.C_ROW, g.C_COL])
+def test_ragged_shapes(dev, M, N, K, b_layout, c_layout):
+    A, Bkn = o.make_inputs(M, N, K, seed=M + 3 * N + 7 * K)
+    got = run_abi(A, layouts(Bkn, b_layout), dev, b_layout, c_layout)
+    o.assert_parity(got, A, Bkn, what=f"{M}x{N}x{K} b{b_layout} c{c_layout}")
+
+
+@pytest.mark.parametrize("variant", TILE_VARIANTS)
+@pytest.mark.parametrize("M,N,K", [(8, 8, 32), (264, 136, 40), (513, 520, 1032), (250, 1000, 72)])
+def test_ragged_shapes_forced_tile_kernels(dev, variant, M, N, K):
+    A, Bkn = o.make_inputs(M, N, K, seed=5 * M + N)
+    for b_layout in (g.B_KN, g.B_NK):
+        B = layouts(Bkn, b_layout)
+        try:
+            got = run_abi(A, B, dev, b_layout, g.C_ROW, variant)
+        except g.NeoGemmError as e:
+            # an MN-major tile narrower than its image, or N % 8 != 0, is refused, never mis-run
+            assert e.status == _abi.ERR_UNSUPPORTED and b_layout == g.B_KN
+            continue
+        o.assert_parity(got, A, Bkn, what=f"{M}x{N}x{K} v{variant} b{b_layout}")
+
+
+def test_k_zero_writes_zeros(dev):
+    A = torch.zeros(5, 0, dtype=torch.bfloat16, device=dev)
+    B = torch.zeros(0, 9, dtype=torch.bfloat16, device=dev)
+    C = g.gemm(A, B)
+    assert C.shape == (5, 9) and torch.all(C == 0)
+
+
+def test_empty_outputs(dev):
+    A = torch.zeros(0, 8, dtype=torch.bfloat16, device=dev)
+    B = torch.zeros(8, 4, dtype=torch.bfloat16, device=dev)
+    assert g.gemm(A, B).shape == (0, 4)
+    A2 = torch.zeros(4, 8, dtype=torch.bfloat16, device=dev)
+    assert g.gemm(A2, B[:, :0]).shape == (4, 0)
+
+
+def test_strided_and_unaligned_operands(dev):
+    M, N, K = 96, 160, 256
+    A, Bkn = o.make_inputs(M, N, K, seed=31)
+    ref = o.ref_gemm(A, Bkn)
+    # leading dimensions larger than the row length (views into wider buffers): MFMA path
+    Aw = torch.zeros(M, K + 64, dtype=torch.bfloat16, device=dev)
+    Aw[:, :K] = A.to(dev)
+    Bw = torch.zeros(K, N + 32, dtype=torch.bfloat16, device=dev)
+    Bw[:, :N] = Bkn.to(dev)
+    o.assert_parity(g.gemm(Aw[:, :K], Bw[:, :N]), A, Bkn, ref=ref, what="wide ld")
+    # base pointers off 16-byte alignment: generic path
+    flatA = torch.zeros(M * K + 8, dtype=torch.bfloat16, device=dev)
+    Au = flatA[3:3 + M * K].view(M, K)
+    Au.copy_(A.to(dev))
+    o.assert_parity(g.gemm(Au, Bkn.to(dev)), A, Bkn, ref=ref, what="unaligned A")
+    # B given as the transposed view of an [N,K] tensor: taken as the reference's layout, no copy
+    Bnk = Bkn.t().contiguous().to(dev)
+    o.assert_parity(g.gemm(A.to(dev), Bnk.t()), A, Bkn, ref=ref, what="B = W.t()")
+    # a column-sliced (non-contiguous rows) A is made contiguous by the wrapper
+    o.assert_parity(g.gemm(Aw.t()[:K].t(), Bkn.to(dev)), A, Bkn, ref=ref, what="A view")
+
+
+# ------------------------------------------------------------------------------------------------
+# the reference's own call, as benchmark.py makes it
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("modname", ["gemm_amd", "neoGEMM"])
+def test_reference_call_contract(dev, modname):
+    """benchmark.py:10-25 with seeded inputs: C = zeros(M,N); neoGemmV1(A, B, C); C.t() == A @ B.t()."""
+    mod = __import__(modname)
+    M = N = K = 1024                                       # benchmark.py:6-8
+    A, Bnk = o.make_inputs(M, N, K, seed=77, b_layout="nk")
+    Ad, Bd = A.to(dev), Bnk.to(dev)
+    C = torch.zeros(M, N, device=dev).to(torch.bfloat16)   # benchmark.py:12
+    assert mod.neoGemmV1(A=Ad, B=Bd, C=C) is None          # keyword names of the binding, returns None
+    torch.cuda.synchronize()
+    o.assert_parity(C.t(), A, Bnk, b_layout="nk", what=f"{modname}.neoGemmV1")
+    C2 = torch.zeros(M, N, device=dev).to(torch.bfloat16)
+    mod.neogemm(Ad, Bd, C2)                                # the older module's name (v01.cu:314-317)
+    torch.cuda.synchronize()
+    assert torch.equal(C2, C)
+    # non-square: the buffer is the column-major product, i.e. an [N,M] row-major matrix
+    M2, N2 = 320, 192
+    A2, B2 = o.make_inputs(M2, N2, K, seed=78, b_layout="nk")
+    C3 = torch.zeros(M2 * N2, device=dev).to(torch.bfloat16).view(M2, N2)
+    mod.neoGemmV1(A2.to(dev), B2.to(dev), C3)
+    torch.cuda.synchronize()
+    o.assert_parity(C3.view(N2, M2).t(), A2, B2, b_layout="nk", what=f"{modname}.neoGemmV1 non-square")
+
+
+def test_module_gemm_matches_abi(dev):
+    import neoGEMM
+    for M, N, K in ((512, 512, 512), (200, 328, 136), (16, 14336, 4096)):
+        A, B = o.make_inputs(M, N, K, seed=M)
+        Ad, Bd = A.to(dev), B.to(dev)
+        C1, C2 = neoGEMM.gemm(Ad, Bd), g.gemm(Ad, Bd)
+        torch.cuda.synchronize()
+        assert C1.dtype == torch.bfloat16 and C1.shape == (M, N) and C1.is_contiguous()
+        assert torch.equal(C1, C2)
+        o.assert_parity(C1, A, B, what=f"neoGEMM.gemm {M}x{N}x{K}")
+    with pytest.raises(RuntimeError, match="inner dimensions"):
+        neoGEMM.gemm(Ad, Ad)
+    with pytest.raises(RuntimeError, match="bfloat16"):
+        neoGEMM.gemm(Ad.float(), Bd.float())
+    with pytest.raises(RuntimeError, match="M\\*N"):
+        neoGEMM.neoGemmV1(Ad, Ad, torch.zeros(3, 3, dtype=torch.bfloat16, device=dev))
+
+
+# ------------------------------------------------------------------------------------------------
+# size-independent properties at full size
+# ------------------------------------------------------------------------------------------------
+def test_properties_full_size(dev):
+    M = N = K = 4096
+    A, B = o.make_inputs(M, N, K, seed=9)
+    Ad, Bd = A.to(dev), B.to(dev)
+    C = g.gemm(Ad, Bd)
+    # deterministic: the same call gives the same bits
+    assert torch.equal(C, g.gemm(Ad, Bd))
+    # scaling by a power of two is exact in every partial sum
+    assert torch.equal(g.gemm((Ad.float() * 4).bfloat16(), Bd), (C.float() * 4).bfloat16())
+    assert torch.equal(g.gemm(Ad, (Bd.float() * 0.5).bfloat16()), (C.float() * 0.5).bfloat16())
+    # (negating an operand is NOT asserted to negate the result bit for bit: the matrix cores' internal
+    # adder is not sign-symmetric in its last bit, so -A gives results 1 ulp apart on a few elements)
+    o.assert_parity(g.gemm(-Ad, Bd)[:64], -A[:64], B, what="negated A")
+    # permuting rows of A permutes rows of C; permuting columns of B permutes columns of C (the
+    # k-order of every dot product does not depend on where its output lies)
+    perm = torch.randperm(M, generator=torch.Generator().manual_seed(1)).to(dev)
+    assert torch.equal(g.gemm(Ad[perm], Bd), C[perm])
+    assert torch.equal(g.gemm(Ad, Bd[:, perm].contiguous()), C[:, perm])
+    # transposition identity: (A B)^T = B^T A^T, computed through the other layout flags
+    Ct = torch.empty(N, M, dtype=torch.bfloat16, device=dev)
+    g.gemm_into(Ad, Bd, Ct, M, N, K, K, N, M, g.B_KN, g.C_COL)
+    assert torch.equal(Ct.t(), C)
+    # checksum of checksums: sum over rows of C equals (1^T A) B up to the rounding of C itself
+    ones_A = Ad.float().sum(0)                       # [K]
+    lhs = C.float().sum(0).double()
+    rhs = (ones_A.double() @ Bd.double())
+    tol = 4.0 * math.sqrt(M) * 2.0 ** -9 * float(C.float().abs().mean()) * 4
+    assert float((lhs - rhs).abs().max()) <= tol * math.sqrt(M)
+
+
+def test_variants_agree_bitwise_on_exact_data(dev):
+    rng = np.random.default_rng(5)
+    M, N, K = 512, 768, 384
+    A = torch.from_numpy(rng.integers(-4, 5, size=(M, K)).astype(np.float32)).to(torch.bfloat16)
+    B = torch.from_numpy(rng.integers(-4, 5, size=(K, N)).astype(np.float32)).to(torch.bfloat16)
+    base = run_abi(A, B, dev, variant=g.VARIANT_GENERIC)
+    for v in TILE_VARIANTS:
+        for gm in (1, 3, 8):
+            assert torch.equal(run_abi(A, B, dev, variant=v, group_m=gm), base)
+
+
+# ------------------------------------------------------------------------------------------------
+# ABI behaviour on the device
+# ------------------------------------------------------------------------------------------------
+def test_error_codes_on_device(dev):
+    M, N, K = 256, 256, 4096
+    A = torch.zeros(M, K, dtype=torch.bfloat16, device=dev)
+    B = torch.zeros(K, N, dtype=torch.bfloat16, device=dev)
+    C = torch.zeros(M, N, dtype=torch.bfloat16, device=dev)
+    ws = torch.zeros(1024, dtype=torch.uint8, device=dev)
+    # split-K without enough workspace
+    st = _abi.gemm_raw(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, K, N, N, 0, 0, ws.data_ptr(), 1024, 0,
+                       g.VARIANT_T128x128_W4, 4, 0)
+    assert st == _abi.ERR_WORKSPACE
+    st = _abi.gemm_raw(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, K, N, N, 0, 0, 0, 0, 0,
+                       g.VARIANT_T128x128_W4, 4, 0)
+    assert st == _abi.ERR_WORKSPACE
+    # a tile kernel asked to run an unaligned problem
+    st = _abi.gemm_raw(A.data_ptr() + 2, B.data_ptr(), C.data_ptr(), M, N, K - 8, K, N, N, 0, 0, 0, 0, 0,
+                       g.VARIANT_T128x128_W4, 1, 0)
+    assert st == _abi.ERR_UNSUPPORTED
+    torch.cuda.synchronize()
+
+
+def test_runs_on_the_callers_stream(dev):
+    A, B = o.make_inputs(512, 512, 1024, seed=4)
+    Ad, Bd = A.to(dev), B.to(dev)
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        C = g.gemm(Ad, Bd)
+        import neoGEMM
+        C2 = neoGEMM.gemm(Ad, Bd)
+    s.synchronize()
+    o.assert_parity(C, A, B, what="side stream")
+    assert torch.equal(C, C2)
+
+
+def test_profile_entry_point(dev):
+    lib = _abi.load()
+    M = N = K = 1024
+    A, B = o.make_inputs(M, N, K, seed=12)
+    Ad, Bd = A.to(dev), B.to(dev)
+    C = torch.zeros(M, N, dtype=torch.bfloat16, device=dev)
+    for variant, waves in ((g.VARIANT_T256x256_W8, 8), (g.VARIANT_T256x256_W4, 4)):
+        nb = lib.neogemm_bf16_profile_bytes(M, N, variant)
+        buf = torch.zeros(nb // 8, dtype=torch.int64, device=dev)
+        st = lib.neogemm_bf16_profile(Ad.data_ptr(), Bd.data_ptr(), C.data_ptr(), M, N, K, K, N, N, 0, None, variant, 0,
+                                      buf.data_ptr(), nb)
+        assert st == 0
+        torch.cuda.synchronize()
+        p = buf.cpu().view(-1, 4)
+        assert p.shape[0] == 16 * waves
+        assert torch.all(p[:, 0] > 0) and torch.all(p[:, 0] >= p[:, 1] + p[:, 2])
+        o.assert_parity(C, A, B, what="profiled run")
+        assert lib.neogemm_bf16_profile(Ad.data_ptr(), Bd.data_ptr(), C.data_ptr(), M, N, K, K, N, N, 0, None, variant, 0,
+                                        buf.data_ptr(), 8) == _abi.ERR_WORKSPACE
