@@ -29,7 +29,10 @@ typedef __attribute__((ext_vector_type(8))) short i16x8;
 #define NEOGEMM_AS3 __attribute__((address_space(3)))
 
 static constexpr int KT = 32;                        // K depth of one LDS slab (bf16 elements)
-static constexpr int NSLAB = 4;                      // slabs in the LDS ring
+#ifndef NEOGEMM_NSLAB
+#define NEOGEMM_NSLAB 4
+#endif
+static constexpr int NSLAB = NEOGEMM_NSLAB;          // slabs in the LDS ring
 static constexpr uint32_t OOB_OFFSET = 0x80000000u;  // >= every num_records this file builds
 
 // ---------------------------------------------------------------------------------------------
@@ -71,7 +74,9 @@ __device__ __forceinline__ void dma_set_m0(uint32_t lds) {
 template <int OFF>
 __device__ __forceinline__ void dma16(i32x4 rsrc, uint32_t voff) {
   static_assert(OFF >= 0 && OFF < 4096, "12-bit instruction offset");
-  asm volatile("buffer_load_dwordx4 %0, %1, 0 offen offset:%2 lds" : : "v"(voff), "s"(rsrc), "n"(OFF) : "memory");
+  // sc1: device-scope load, i.e. do not keep the line in the CU's 32 KiB vector L1 — the data goes
+  // straight to LDS and is never re-read through L1; measured +4.6 % on N(0,1) data at 8192^3.
+  asm volatile("buffer_load_dwordx4 %0, %1, 0 offen offset:%2 sc1 lds" : : "v"(voff), "s"(rsrc), "n"(OFF) : "memory");
 }
 
 // acc += A(16x32) * B(32x16) with the accumulator pinned in AGPRs and written in place.  Written as
@@ -296,7 +301,7 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
   constexpr int HM = TM / 2;
   bf16x8 af[TM], bfr[TN];  // one copy of each fragment; refreshed in place as soon as it is dead
 
-  auto img_of = [&](int slab) -> uint32_t { return lds0 + (uint32_t)(slab & (NSLAB - 1)) * SLAB; };
+  auto img_of = [&](int slab) -> uint32_t { return lds0 + (uint32_t)(slab % NSLAB) * SLAB; };
 
   // Half a slab step: the MFMAs of fragment rows [HALF*HM, HALF*HM + HM) against every B fragment,
   // column by column, with the LDS reads that refresh dead fragments and (DMA) this wave's loads of
@@ -420,11 +425,11 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
 
   int j = 0;
   // steady: slab j+4 exists and is not the last one (the last may need its K tail masked)
-  for (; j + 3 + NSLAB < nslab - 1; j += NSLAB) {
+  for (; j + (NSLAB - 1) + NSLAB < nslab - 1; j += NSLAB) {
 #pragma unroll
     for (int u = 0; u < NSLAB; ++u) {
-      const uint32_t img_free = lds0 + u * SLAB, img_next = lds0 + ((u + 1) & (NSLAB - 1)) * SLAB;
-      sync(std::integral_constant<int, 2 * LPS>{});
+      const uint32_t img_free = lds0 + u * SLAB, img_next = lds0 + ((u + 1) % NSLAB) * SLAB;
+      sync(std::integral_constant<int, (NSLAB - 2) * LPS>{});
       half_step(H1{}, T{}, img_next, T{}, img_free);
       half_step(H0{}, T{}, img_next, T{}, img_free);
     }
@@ -453,7 +458,57 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
 
   // Epilogue: lane holds, per 16x16 tile, output row (lane & 15) and 4 consecutive columns 4*(lane >> 4)..+3.
   const int row_l = lane & 15, colq = (lane >> 4) * 4;
-  if (p.ksplit == 1) {
+  // Coalesced path: the wave parks its bf16 tile in LDS (the slab ring is dead by now) and reads it back
+  // row-wise, so that a store instruction writes whole rows of the wave tile, 16 bytes per lane, instead of
+  // sixteen 32-byte pieces.  The staging tile is WTM x WTN bf16, 16-byte chunks XOR-ed with the row number
+  // so that neither the 8-byte writes (16 rows per instruction) nor the 16-byte reads collide on banks.
+  constexpr int CH = WTN / 8;        // 16-byte chunks per staged row
+  constexpr int RPI = 64 / CH;       // rows one store instruction covers
+  constexpr bool CAN_STAGE = (size_t)BM * BN * 2 <= (size_t)NSLAB * SLAB && CH >= 4 && CH <= 64;
+  const bool stage = CAN_STAGE && p.ksplit == 1 && (((uintptr_t)p.C | (uintptr_t)(p.ldc * 2)) & 15) == 0;
+  if (stage) {
+    if constexpr (CAN_STAGE) {
+      // every wave is done with the slab images (its LDS reads have returned: the MFMAs that used them
+      // were issued; wait anyway) before any wave overwrites them
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+      const uint32_t region = lds0 + (uint32_t)wave * (WTM * WTN * 2);
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        const uint32_t row = i * 16 + row_l;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          bf16x4 o;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) o[r] = (__bf16)acc[i][j][r];
+          const uint32_t c = 2 * j + (lane >> 5);
+          const uint32_t addr = region + row * (WTN * 2) + ((c ^ (row & (CH - 1))) << 4) + (((lane >> 4) & 1) << 3);
+          *((NEOGEMM_AS3 bf16x4*)(uintptr_t)addr) = o;
+        }
+      }
+      // same wave wrote and reads: LDS operations of a wave complete in order; the compiler orders them
+      const int colc = lane % CH;
+      const int col = n0 + wn * WTN + colc * 8;
+#pragma unroll
+      for (int st = 0; st < WTM / RPI; ++st) {
+        const uint32_t row = st * RPI + lane / CH;
+        const uint32_t addr = region + row * (WTN * 2) + (((uint32_t)colc ^ (row & (CH - 1))) << 4);
+        const bf16x8 v = *((NEOGEMM_AS3 bf16x8*)(uintptr_t)addr);
+        const int grow = m0 + wm * WTM + (int)row;
+        if (grow < p.M) {
+          char* dst = p.C + ((size_t)grow * p.ldc + col) * 2;
+          if (col + 7 < p.N) {
+            *(bf16x8*)dst = v;
+          } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+              if (col + e < p.N) ((__bf16*)dst)[e] = v[e];
+          }
+        }
+      }
+    }
+  } else if (p.ksplit == 1) {
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
       const int row = m0 + wm * WTM + i * 16 + row_l;
