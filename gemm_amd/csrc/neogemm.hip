@@ -663,24 +663,38 @@ static bool is_aligned(const void* A, const void* B, const void* C, int64_t K, i
 static int ceil_div(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
 
 // Shape -> (variant, split_k).  256 CUs; a 256x256 workgroup fills one CU (128 KiB of LDS).
-static void plan(int64_t M, int64_t N, int64_t K, bool aligned, int* variant, int* split_k) {
+// (M, N) as the caller states them; c_layout tells which of the two the kernel will see as its rows.
+static void plan(int64_t M, int64_t N, int64_t K, bool aligned, int c_layout, int* variant, int* split_k) {
   if (!aligned || K == 0) {
     *variant = NEOGEMM_VARIANT_GENERIC;
     *split_k = 1;
     return;
   }
-  // One wave per SIMD with a 128x128 wave tile reads the least LDS per flop; below ~64 such tiles the
-  // 128x128 macro-tile (4 per CU's worth of work) fills the chip better.
-  int v = NEOGEMM_VARIANT_T256x256_W4;
-  if (M <= 128 || N <= 128 || (int64_t)ceil_div(M, 256) * ceil_div(N, 256) < 64) v = NEOGEMM_VARIANT_T128x128_W4;
-  const int64_t tiles = (int64_t)ceil_div(M, kVariants[v].bm) * ceil_div(N, kVariants[v].bn);
+  const int64_t rows = c_layout == NEOGEMM_C_ROW ? M : N, cols = c_layout == NEOGEMM_C_ROW ? N : M;
   const int64_t ktiles = ceil_div(K, KT);
+  int v, slots;  // slots: workgroups of this variant the 256 CUs hold at once (LDS-limited)
+  if ((int64_t)ceil_div(rows, 256) * ceil_div(cols, 256) >= 64 && rows > 128 && cols > 128) {
+    // One wave per SIMD with a 128x128 wave tile reads the least LDS per flop.
+    v = NEOGEMM_VARIANT_T256x256_W4;
+    slots = 256;
+  } else if (rows <= 128 && cols >= 2048) {
+    // skinny, streaming the wide operand: 128x256 tiles keep the most bytes in flight per workgroup
+    v = NEOGEMM_VARIANT_T128x256_W8;
+    slots = 256;
+  } else if (cols <= 128 && rows >= 2048) {
+    v = NEOGEMM_VARIANT_T256x128_W8;
+    slots = 256;
+  } else {
+    v = NEOGEMM_VARIANT_T128x128_W4;
+    slots = 512;
+  }
+  const int64_t tiles = (int64_t)ceil_div(rows, kVariants[v].bm) * ceil_div(cols, kVariants[v].bn);
   int s = 1;
-  if (tiles < 192) {
-    // not enough tiles to fill the chip: split K until there are ~2 workgroups per CU, keeping >= 4
-    // K tiles per split so the pipeline has something to overlap
-    int64_t want = (512 + tiles - 1) / tiles;
-    int64_t maxs = ktiles / 4 > 0 ? ktiles / 4 : 1;
+  if (tiles * 4 < slots * 3) {
+    // not enough tiles to fill the chip: split K so that one round of workgroups covers the CUs,
+    // keeping >= 8 slabs per split so the pipeline has something to overlap
+    int64_t want = slots / tiles;
+    int64_t maxs = ktiles / 8 > 0 ? ktiles / 8 : 1;
     s = (int)(want < maxs ? want : maxs);
     if (s < 1) s = 1;
     if (s > 64) s = 64;
@@ -708,7 +722,7 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
   int v = variant, s = split_k;
   if (v == NEOGEMM_VARIANT_AUTO) {
     int pv, ps;
-    plan(M, N, K, aligned, &pv, &ps);
+    plan(M, N, K, aligned, c_layout, &pv, &ps);
     v = pv;
     if (s == 0) s = ps;
   }
@@ -754,8 +768,14 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
                     (bk ? a.ldb >= 32 : (vi.bn >= 128 && a.ldb >= vi.bn && (a.N & 7) == 0));
   if (!fits) {
     if (variant != NEOGEMM_VARIANT_AUTO) return NEOGEMM_ERR_UNSUPPORTED;
-    return run(A, B, C, M, N, K, lda, ldb, ldc, b_layout, c_layout, workspace, workspace_bytes, hip_stream,
+    // the planned tile is too wide for an MN-major operand: the 128x128 tile needs the least, then generic
+    const int next = v != NEOGEMM_VARIANT_T128x128_W4 ? NEOGEMM_VARIANT_T128x128_W4 : NEOGEMM_VARIANT_GENERIC;
+    int st = run(A, B, C, M, N, K, lda, ldb, ldc, b_layout, c_layout, workspace, workspace_bytes, hip_stream, next,
+                 next == NEOGEMM_VARIANT_GENERIC ? 1 : s, 0, nullptr);
+    if (st == NEOGEMM_ERR_UNSUPPORTED && next != NEOGEMM_VARIANT_GENERIC)
+      st = run(A, B, C, M, N, K, lda, ldb, ldc, b_layout, c_layout, workspace, workspace_bytes, hip_stream,
                NEOGEMM_VARIANT_GENERIC, 1, 0, nullptr);
+    return st;
   }
   a.ntm = ceil_div(a.M, vi.bm);
   a.ntn = ceil_div(a.N, vi.bn);
@@ -837,16 +857,20 @@ size_t neogemm_bf16_profile_bytes(int64_t M, int64_t N, int variant) {
 size_t neogemm_bf16_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   if (M <= 0 || N <= 0 || K <= 0) return 0;
   int v, s;
-  neogemm::plan(M, N, K, true, &v, &s);
+  // the larger of the two output layouts' needs, so that one query covers any call for this shape
+  int v2, s2;
+  neogemm::plan(M, N, K, true, NEOGEMM_C_ROW, &v, &s);
+  neogemm::plan(M, N, K, true, NEOGEMM_C_COL, &v2, &s2);
+  if (s2 > s) s = s2;
   return s > 1 ? (size_t)s * (size_t)M * (size_t)N * sizeof(float) : 0;
 }
 
 int neogemm_bf16_plan(int64_t M, int64_t N, int64_t K, int b_layout, int c_layout, int aligned, int* variant,
                       int* split_k) {
   (void)b_layout;
-  (void)c_layout;
   if (!variant || !split_k || M < 0 || N < 0 || K < 0) return NEOGEMM_ERR_BAD_ARG;
-  neogemm::plan(M, N, K, aligned != 0, variant, split_k);
+  if (c_layout != NEOGEMM_C_ROW && c_layout != NEOGEMM_C_COL) return NEOGEMM_ERR_BAD_ARG;
+  neogemm::plan(M, N, K, aligned != 0, c_layout, variant, split_k);
   return NEOGEMM_OK;
 }
 
