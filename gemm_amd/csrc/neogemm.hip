@@ -323,31 +323,33 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
     }
     static_for<TN>([&](auto cc) {
       constexpr int c = decltype(cc)::value;
-#pragma unroll
-      for (int i = HALF * HM; i < HALF * HM + HM; ++i)
+      constexpr int a_lo = c * APC < HM ? c * APC : HM, a_hi = (c + 1) * APC < HM ? (c + 1) * APC : HM;
+      constexpr int l_lo = c * NL / TN, l_hi = (c + 1) * NL / TN;  // loads: NL of them spread over the TN columns
+      // Column c: HM MFMAs.  At most one memory instruction goes between two MFMAs: the A refreshes
+      // after the first MFMA, the direct-to-LDS load after the second, the B refresh after the last
+      // (which is the last reader of bfr[c]).
+      static_for<HM>([&](auto ic) {
+        constexpr int ii = decltype(ic)::value;
+        constexpr int i = HALF * HM + ii;
         // B fragment first: D rows index n, D columns index m, so a lane ends up with 4
         // consecutive n of one output row (an 8-byte store) instead of 4 rows of one column.
         mfma_16x16x32(acc[i][c], bfr[c], af[i]);
-      constexpr int a_lo = c * APC < HM ? c * APC : HM, a_hi = (c + 1) * APC < HM ? (c + 1) * APC : HM;
-      constexpr int nread = READ ? (a_hi - a_lo) * (AK ? 1 : 2) + (HALF == 1 ? (BK ? 1 : 2) : 0) : 0;
-      if constexpr (READ) {
-        if constexpr (HALF == 1) bfr[c] = fb.read(img_rd + A_BYTES, c);
+        if constexpr (READ && ii == 0) {
 #pragma unroll
-        for (int f = a_lo; f < a_hi; ++f) {
-          if constexpr (HALF == 0) af[HM + f] = fa.read(img_rd, HM + f);
-          else af[f] = fa.read(img_rd, f);
+          for (int f = a_lo; f < a_hi; ++f) {
+            if constexpr (HALF == 0) af[HM + f] = fa.read(img_rd, HM + f);
+            else af[f] = fa.read(img_rd, f);
+          }
         }
-      }
-      (void)nread;
-      // loads: NL of them spread over the TN columns
-      constexpr int l_lo = c * NL / TN, l_hi = (c + 1) * NL / TN;
-      if constexpr (l_hi > l_lo) {
-        static_for<l_hi - l_lo>([&](auto lc) {
-          constexpr int l = l_lo + decltype(lc)::value;
-          if constexpr (HALF == 1) opa.template issue_one<l>(rs);
-          else opb.template issue_one<l>(rs);
-        });
-      }
+        if constexpr (ii == (HM > 1 ? 1 : 0) && l_hi > l_lo) {
+          static_for<l_hi - l_lo>([&](auto lc) {
+            constexpr int l = l_lo + decltype(lc)::value;
+            if constexpr (HALF == 1) opa.template issue_one<l>(rs);
+            else opb.template issue_one<l>(rs);
+          });
+        }
+      });
+      if constexpr (READ && HALF == 1) bfr[c] = fb.read(img_rd + A_BYTES, c);
     });
     if constexpr (DMA) {
       if constexpr (HALF == 1) opa.advance();
