@@ -41,8 +41,8 @@ static constexpr uint32_t OOB_OFFSET = 0x80000000u;  // >= every num_records thi
 // K-major operand (rows of the matrix are K-contiguous: A[M,K], B[N,K]):
 //   image = ROWS x 64 B, row r at r*64, four 16-byte chunks per row; logical chunk c of row r lives
 //   at physical chunk c ^ swz_k(r).  An MFMA operand read (16 rows x 32 k) has 16 lanes fetch the
-//   same logical chunk of 16 consecutive rows; swz_k makes any 8 consecutive rows cover the 8 slots
-//   of a 128-byte window and any 16 consecutive rows the 16 slots of a 256-byte window exactly once.
+//   same logical chunk of 16 consecutive rows; swz_k spreads them over the banks (chosen by timing
+//   every XOR-linear candidate on the hardware, see swz_k).
 // MN-major operand (the K index is the slow one: B[K,N]):
 //   image = 32 x (ROWS*2) B, k-row at k*ROWS*2; logical chunk c (8 columns) of k-row k lives at
 //   physical chunk c ^ swz_mn(k).  Read back with ds_read_b64_tr_b16: in each group of 16 lanes,
@@ -53,7 +53,10 @@ static constexpr uint32_t OOB_OFFSET = 0x80000000u;  // >= every num_records thi
 // global chunk each lane fetches.
 // ---------------------------------------------------------------------------------------------
 __device__ __forceinline__ uint32_t swz_k(uint32_t row) {
-  return (((row >> 2) & 1u) << 1) | (((row >> 1) ^ (row >> 3)) & 1u);
+  // bit 0 = row bit 1, bit 1 = row bit 1 ^ row bit 2: the fastest of the 256 XOR-linear 2-bit functions of
+  // the row number for the 16-row x 4-chunk ds_read_b128 pattern, timed on the hardware (211 B/clk/CU;
+  // no swizzle: 130)
+  return ((row >> 1) & 1u) | ((((row >> 1) ^ (row >> 2)) & 1u) << 1);
 }
 __device__ __forceinline__ uint32_t swz_mn(uint32_t krow) {
   // even values 0..14: (k & 3) picks the 32-byte pair, bit 3 of k the 128-byte half
