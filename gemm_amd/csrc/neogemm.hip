@@ -29,10 +29,6 @@ typedef __attribute__((ext_vector_type(8))) short i16x8;
 #define NEOGEMM_AS3 __attribute__((address_space(3)))
 
 static constexpr int KT = 32;                        // K depth of one LDS slab (bf16 elements)
-#ifndef NEOGEMM_NSLAB
-#define NEOGEMM_NSLAB 4
-#endif
-static constexpr int NSLAB = NEOGEMM_NSLAB;          // slabs in the LDS ring
 static constexpr uint32_t OOB_OFFSET = 0x80000000u;  // >= every num_records this file builds
 
 // ---------------------------------------------------------------------------------------------
@@ -239,7 +235,7 @@ struct FragReader {
 // PROF adds s_memtime stamps around the two waits of the main loop and writes, per wave,
 // {total, waiting for own loads, waiting at the barrier, epilogue} shader-clock cycles to p.prof — the
 // per-phase cycle buffer idea of the reference's harness (cublass/matmul.cu:99-106,149-165).
-template <int BM, int BN, int WGM, int WGN, bool AK, bool BK, bool PROF = false>
+template <int BM, int BN, int WGM, int WGN, int NSLAB, bool AK, bool BK, bool PROF = false>
 __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
   constexpr int NW = WGM * WGN;
   constexpr int WTM = BM / WGM, WTN = BN / WGN;
@@ -625,10 +621,10 @@ struct VariantInfo {
   int bm, bn, nwaves;
 };
 static const VariantInfo kVariants[NEOGEMM_VARIANT_COUNT] = {
-    {0, 0, 0}, {16, 16, 4}, {256, 256, 8}, {256, 256, 4}, {128, 128, 4}, {256, 128, 8}, {128, 256, 8},
+    {0, 0, 0}, {16, 16, 4}, {256, 256, 8}, {256, 256, 4}, {128, 128, 4}, {256, 128, 8}, {128, 256, 8}, {64, 128, 4}, {128, 128, 4},
 };
 
-template <int BM, int BN, int WGM, int WGN>
+template <int BM, int BN, int WGM, int WGN, int NSLAB>
 static hipError_t launch_tile(const TileArgs& a, bool ak, bool bk, hipStream_t st) {
   constexpr size_t lds = (size_t)NSLAB * (BM + BN) * KT * 2;
   dim3 grid(a.ntm * a.ntn, a.ksplit), block(WGM * WGN * 64);
@@ -644,17 +640,17 @@ static hipError_t launch_tile(const TileArgs& a, bool ak, bool bk, hipStream_t s
   };
   if (a.prof) {
     if constexpr (BM == 256 && BN == 256) {
-      if (ak && bk) return go(gemm_tile_kernel<BM, BN, WGM, WGN, true, true, true>);
-      if (ak && !bk) return go(gemm_tile_kernel<BM, BN, WGM, WGN, true, false, true>);
+      if (ak && bk) return go(gemm_tile_kernel<BM, BN, WGM, WGN, NSLAB, true, true, true>);
+      if (ak && !bk) return go(gemm_tile_kernel<BM, BN, WGM, WGN, NSLAB, true, false, true>);
     }
     return hipErrorInvalidValue;
   }
-  if (ak && bk) return go(gemm_tile_kernel<BM, BN, WGM, WGN, true, true>);
+  if (ak && bk) return go(gemm_tile_kernel<BM, BN, WGM, WGN, NSLAB, true, true>);
   if (ak && !bk) {
-    if constexpr (BN >= 128) return go(gemm_tile_kernel<BM, BN, WGM, WGN, true, false>);
+    if constexpr (BN >= 128) return go(gemm_tile_kernel<BM, BN, WGM, WGN, NSLAB, true, false>);
   }
   if (!ak && bk) {
-    if constexpr (BM >= 128) return go(gemm_tile_kernel<BM, BN, WGM, WGN, false, true>);
+    if constexpr (BM >= 128) return go(gemm_tile_kernel<BM, BN, WGM, WGN, NSLAB, false, true>);
   }
   return hipErrorInvalidValue;
 }
@@ -802,11 +798,13 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
 
   hipError_t e;
   switch (v) {
-    case NEOGEMM_VARIANT_T256x256_W8: e = launch_tile<256, 256, 2, 4>(a, ak, bk, st); break;
-    case NEOGEMM_VARIANT_T256x256_W4: e = launch_tile<256, 256, 2, 2>(a, ak, bk, st); break;
-    case NEOGEMM_VARIANT_T128x128_W4: e = launch_tile<128, 128, 2, 2>(a, ak, bk, st); break;
-    case NEOGEMM_VARIANT_T256x128_W8: e = launch_tile<256, 128, 4, 2>(a, ak, bk, st); break;
-    case NEOGEMM_VARIANT_T128x256_W8: e = launch_tile<128, 256, 2, 4>(a, ak, bk, st); break;
+    case NEOGEMM_VARIANT_T256x256_W8: e = launch_tile<256, 256, 2, 4, 4>(a, ak, bk, st); break;
+    case NEOGEMM_VARIANT_T256x256_W4: e = launch_tile<256, 256, 2, 2, 4>(a, ak, bk, st); break;
+    case NEOGEMM_VARIANT_T128x128_W4: e = launch_tile<128, 128, 2, 2, 4>(a, ak, bk, st); break;
+    case NEOGEMM_VARIANT_T256x128_W8: e = launch_tile<256, 128, 4, 2, 4>(a, ak, bk, st); break;
+    case NEOGEMM_VARIANT_T128x256_W8: e = launch_tile<128, 256, 2, 4, 4>(a, ak, bk, st); break;
+    case NEOGEMM_VARIANT_T64x128_W4: e = launch_tile<64, 128, 1, 4, 6>(a, ak, bk, st); break;
+    case NEOGEMM_VARIANT_T128x128_W4S: e = launch_tile<128, 128, 1, 4, 5>(a, ak, bk, st); break;
     default: return NEOGEMM_ERR_BAD_ARG;
   }
   if (e != hipSuccess) {

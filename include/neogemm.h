@@ -47,7 +47,9 @@ extern "C" {
 #define NEOGEMM_VARIANT_T128x128_W4 4 /* 128x128x64 macro-tile, 4 wave64 (2x2) */
 #define NEOGEMM_VARIANT_T256x128_W8 5 /* 256x128x64 macro-tile, 8 wave64 (4x2) */
 #define NEOGEMM_VARIANT_T128x256_W8 6 /* 128x256x64 macro-tile, 8 wave64 (2x4) */
-#define NEOGEMM_VARIANT_COUNT 7
+#define NEOGEMM_VARIANT_T64x128_W4 7  /* 64x128x32 macro-tile, 4 wave64 (1x4), 6-slab ring: streaming, M <= 64 */
+#define NEOGEMM_VARIANT_T128x128_W4S 8 /* 128x128x32 macro-tile, 4 wave64 (1x4), 5-slab ring: streaming, M <= 128 */
+#define NEOGEMM_VARIANT_COUNT 9
 
 /*
  * C = A * op(B), bf16 in, fp32 accumulate, bf16 out.

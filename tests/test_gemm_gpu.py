@@ -22,19 +22,26 @@ from oracle import gemm_oracle as o
 pytestmark = pytest.mark.gpu
 
 TILE_VARIANTS = [g.VARIANT_T256x256_W8, g.VARIANT_T256x256_W4, g.VARIANT_T128x128_W4, g.VARIANT_T256x128_W8,
-                 g.VARIANT_T128x256_W8]
+                 g.VARIANT_T128x256_W8, g.VARIANT_T64x128_W4, g.VARIANT_T128x128_W4S]
 ALL_VARIANTS = [g.VARIANT_GENERIC] + TILE_VARIANTS
 
 
-def run_abi(A, B, dev, b_layout=g.B_KN, c_layout=g.C_ROW, variant=None, split_k=0, group_m=0):
+def run_abi(A, B, dev, b_layout=g.B_KN, c_layout=g.C_ROW, variant=None, split_k=0, group_m=0, strict=False):
     """A [M,K] and B ([K,N] or [N,K]) are CPU bf16 tensors; returns the [M,N] result on the CPU."""
     M, K = A.shape
     N = B.shape[1] if b_layout == g.B_KN else B.shape[0]
     Ad, Bd = A.to(dev), B.to(dev)
     shape = (M, N) if c_layout == g.C_ROW else (N, M)
     C = torch.full(shape, float("nan"), dtype=torch.bfloat16, device=dev)   # poison: every element must be written
-    g.gemm_into(Ad, Bd, C, M, N, K, max(K, 1), max(N if b_layout == g.B_KN else K, 1),
-                max(N if c_layout == g.C_ROW else M, 1), b_layout, c_layout, variant, split_k, group_m)
+    try:
+        g.gemm_into(Ad, Bd, C, M, N, K, max(K, 1), max(N if b_layout == g.B_KN else K, 1),
+                    max(N if c_layout == g.C_ROW else M, 1), b_layout, c_layout, variant, split_k, group_m)
+    except g.NeoGemmError as e:
+        if e.status == _abi.ERR_UNSUPPORTED and variant not in (None, g.VARIANT_GENERIC) and not strict:
+            # a forced tile variant may refuse a layout (an MN-major operand needs a tile >= 128 wide, ld >= tile,
+            # rows % 8 == 0; a K-major one ld >= 32): refusing is the documented behaviour, mis-running would not be
+            pytest.skip(f"variant {variant} refuses this layout/shape (status {e.status})")
+        raise
     torch.cuda.synchronize()
     C = C.cpu()
     return C if c_layout == g.C_ROW else C.t().contiguous()
@@ -194,7 +201,7 @@ def test_ragged_shapes_forced_tile_kernels(dev, variant, M, N, K):
     for b_layout in (g.B_KN, g.B_NK):
         B = layouts(Bkn, b_layout)
         try:
-            got = run_abi(A, B, dev, b_layout, g.C_ROW, variant)
+            got = run_abi(A, B, dev, b_layout, g.C_ROW, variant, strict=True)
         except g.NeoGemmError as e:
             # an MN-major tile narrower than its image, or N % 8 != 0, is refused, never mis-run
             assert e.status == _abi.ERR_UNSUPPORTED and b_layout == g.B_KN
