@@ -28,31 +28,33 @@ typedef __attribute__((ext_vector_type(8))) short i16x8;
 
 #define NEOGEMM_AS3 __attribute__((address_space(3)))
 
-static constexpr int KT = 32;                        // K depth of one LDS slab (bf16 elements)
+static constexpr int KT = 32;                        // K depth of one MFMA step / one slab (bf16 elements)
+static constexpr int KTILE = 64;                     // K depth of a K-major LDS image, and the split-K unit
 static constexpr uint32_t OOB_OFFSET = 0x80000000u;  // >= every num_records this file builds
 
 // ---------------------------------------------------------------------------------------------
-// LDS image of one operand slab (ROWS x 32 k) and its swizzles.
+// LDS images and their swizzles.  K is consumed in slabs of 32 (one v_mfma_f32_16x16x32_bf16 step).
 //
-// K-major operand (rows of the matrix are K-contiguous: A[M,K], B[N,K]):
-//   image = ROWS x 64 B, row r at r*64, four 16-byte chunks per row; logical chunk c of row r lives
-//   at physical chunk c ^ swz_k(r).  An MFMA operand read (16 rows x 32 k) has 16 lanes fetch the
-//   same logical chunk of 16 consecutive rows; swz_k spreads them over the banks (chosen by timing
-//   every XOR-linear candidate on the hardware, see swz_k).
-// MN-major operand (the K index is the slow one: B[K,N]):
-//   image = 32 x (ROWS*2) B, k-row at k*ROWS*2; logical chunk c (8 columns) of k-row k lives at
-//   physical chunk c ^ swz_mn(k).  Read back with ds_read_b64_tr_b16: in each group of 16 lanes,
-//   lanes 4r..4r+3 address k-row r (16 columns, 8 bytes per lane) and lane j receives the 4 k-values
-//   of column j.  A half-wave touches k-rows {0..3} and {8..11} (+4, +16), 32 bytes of each: swz_mn
-//   spreads those eight 32-byte pieces over the 64 banks.
-// Direct-to-LDS loads write 64 lanes x 16 B contiguously, so the swizzle is applied by choosing which
-// global chunk each lane fetches.
+// K-major operand (rows of the matrix are K-contiguous: A[M,K], B[N,K]) — image of a 64-deep TILE:
+//   ROWS x 128 B, row r at r*128, eight 16-byte chunks per row, slab s of the tile in chunks 4s..4s+3;
+//   logical chunk c of row r lives at physical chunk c ^ swz_k(r).  64 deep, not 32, so that one
+//   direct-to-LDS instruction (8 rows x 128 B) asks the L2 for whole 128-byte lines: with 64-byte
+//   pieces the vector L1 issues twice the requests and the wave that issues the load is held up
+//   roughly in proportion to the number of requests.  Two images per operand (double buffer).
+// MN-major operand (the K index is the slow one: B[K,N]) — image of a 32-deep SLAB:
+//   32 x (ROWS*2) B, k-row at k*ROWS*2; logical chunk c (8 columns) of k-row k lives at physical
+//   chunk c ^ swz_mn(k).  Rows are whole lines already.  Read back with ds_read_b64_tr_b16: in each
+//   group of 16 lanes, lanes 4r..4r+3 address k-row r (16 columns, 8 bytes per lane) and lane j
+//   receives the 4 k-values of column j.  A half-wave touches k-rows {0..3} and {8..11} (+4, +16),
+//   32 bytes of each: swz_mn spreads those eight pieces over the 64 banks.  Four images (ring).
+// Either way an operand owns ROWS*256 bytes of LDS.  Direct-to-LDS loads write 64 lanes x 16 B
+// contiguously, so a swizzle is applied by choosing which global chunk each lane fetches.
 // ---------------------------------------------------------------------------------------------
 __device__ __forceinline__ uint32_t swz_k(uint32_t row) {
-  // bit 0 = row bit 1, bit 1 = row bit 1 ^ row bit 2: the fastest of the 256 XOR-linear 2-bit functions of
-  // the row number for the 16-row x 4-chunk ds_read_b128 pattern, timed on the hardware (211 B/clk/CU;
-  // no swizzle: 130)
-  return ((row >> 1) & 1u) | ((((row >> 1) ^ (row >> 2)) & 1u) << 1);
+  // bits: row2 | (row0^row2) << 1 | (row0^row1) << 2 — the fastest of the 4096 XOR-linear 3-bit
+  // functions of the row number for the 16-row x 4-chunk ds_read_b128 pattern, timed on the hardware
+  // (246 B/clk/CU; no swizzle: 77)
+  return ((row >> 2) & 1u) | (((row ^ (row >> 2)) & 1u) << 1) | (((row ^ (row >> 1)) & 1u) << 2);
 }
 __device__ __forceinline__ uint32_t swz_mn(uint32_t krow) {
   // even values 0..14: (k & 3) picks the 32-byte pair, bit 3 of k the 128-byte half
@@ -111,20 +113,24 @@ struct TileArgs {
   int M, N, K;
   long lda, ldb, ldc;  // elements
   int ntm, ntn, group_m;
-  int ksplit, ktiles_per_split;  // K is cut in slabs of KT; a split is a run of slabs
+  int ksplit, ktiles_per_split;  // K is cut in tiles of KTILE; a split is a run of tiles
   unsigned long long* prof;      // phase timers, 4 per wave (profiling instantiation only)
 };
 
 // Global -> LDS side of one operand: which 16 bytes each lane fetches for each of this wave's
-// 1 KiB loads of a slab, and the buffer resource that walks along K.
-template <int ROWS, bool KMAJOR, int NW>
+// 1 KiB loads of a unit (a 64-deep tile if K-major, a 32-deep slab if MN-major), and the buffer
+// resource that walks along K.
+template <int ROWS, bool KMAJOR, int NW, int NIMG>
 struct Operand {
-  static constexpr int NINSTR = ROWS / 16;  // 1 KiB wave-loads per slab
-  static constexpr int IPW = NINSTR / NW;   // per wave
-  static constexpr int ROWB = ROWS * 2;     // bytes per k-row of an MN-major image
-  static constexpr int CPR = ROWS / 8;      // 16-byte chunks per k-row (MN-major)
-  static constexpr int KR = 64 / CPR;       // k-rows per wave-load (MN-major)
-  static_assert(NINSTR % NW == 0 && IPW >= 1 && IPW <= 4, "slab loads must divide evenly over the waves, at most 4 each");
+  static constexpr int UNIT_K = KMAJOR ? KTILE : KT;       // K depth of one unit
+  static constexpr int UNITS = NIMG;                       // images in LDS
+  static constexpr uint32_t IMG = ROWS * UNIT_K * 2;       // bytes per image
+  static constexpr int NINSTR = IMG / 1024;                // 1 KiB wave-loads per unit
+  static constexpr int IPW = NINSTR / NW;                  // per wave
+  static constexpr int ROWB = ROWS * 2;                    // bytes per k-row of an MN-major image
+  static constexpr int CPR = ROWS / 8;                     // 16-byte chunks per k-row (MN-major)
+  static constexpr int KR = 64 / CPR;                      // k-rows per wave-load (MN-major)
+  static_assert(NINSTR % NW == 0 && IPW >= 1 && IPW <= 8, "unit loads must divide evenly over the waves");
   static_assert(KMAJOR || ROWS >= 128, "MN-major swizzle needs >= 16 chunks per k-row");
 
   uint32_t voff[IPW];
@@ -135,18 +141,19 @@ struct Operand {
   // Every lane offset that would leave the matrix is replaced by OOB_OFFSET, which the buffer range
   // check (num_records = 2 GiB, constant) turns into a zero fill without a memory access; all other
   // offsets address bytes inside the matrix, so the resource needs no exact size and only its base
-  // moves along K.
+  // moves along K.  Load j carries the instruction offset (j & 3) * 1024, which moves the global and the
+  // LDS address alike: the lane offsets are biased by it (rows grow faster than the bias, see the host
+  // checks on ld).
   __device__ __forceinline__ void init(const char* ptr, long ld, int rows_total, int r0, int k_begin, int wave,
                                        int lane) {
     if constexpr (KMAJOR) {
       base = (uint64_t)ptr + ((uint64_t)r0 * ld + k_begin) * 2;
-      kadv = KT * 2;
+      kadv = KTILE * 2;
 #pragma unroll
       for (int j = 0; j < IPW; ++j) {
-        uint32_t row = (wave * IPW + j) * 16 + (lane >> 2);
-        uint32_t c = (lane & 3) ^ swz_k(row);
-        // load j carries instruction offset j*1024 (see dma16); row >= 16*j and ld >= 32 keep this >= 0
-        voff[j] = row * (uint32_t)ld * 2 + c * 16 - j * 1024;
+        uint32_t row = (wave * IPW + j) * 8 + (lane >> 3);
+        uint32_t c = (lane & 7) ^ swz_k(row);
+        voff[j] = row * (uint32_t)ld * 2 + c * 16 - (j & 3) * 1024;  // row >= 8*j and ld >= 64 keep this >= 0
         if (r0 + (int)row >= rows_total) voff[j] = OOB_OFFSET;
       }
     } else {
@@ -156,8 +163,7 @@ struct Operand {
       for (int j = 0; j < IPW; ++j) {
         uint32_t krow = (wave * IPW + j) * KR + lane / CPR;
         uint32_t c = (lane % CPR) ^ swz_mn(krow);
-        // krow >= KR*j and ld >= ROWS keep this >= 0
-        voff[j] = krow * (uint32_t)ld * 2 + c * 16 - j * 1024;
+        voff[j] = krow * (uint32_t)ld * 2 + c * 16 - (j & 3) * 1024;  // krow >= KR*j and ld >= ROWS keep this >= 0
         // a chunk past the last column would wrap into the next k-row (rows_total % 8 == 0: no straddling)
         if (r0 + (int)c * 8 >= rows_total) voff[j] = OOB_OFFSET;
       }
@@ -165,14 +171,15 @@ struct Operand {
     lds_w = wave * IPW * 1024;
   }
 
-  // Last, partial slab of depth krem: drop what lies past K (K-major: chunks that would wrap into the
-  // next row; MN-major: whole k-rows).
+  // Drop what lies at or past depth krem of the unit about to be loaded (K-major: chunks, which would
+  // wrap into the next row; MN-major: whole k-rows).  krem may be <= 0 (a unit entirely past K).
+  // Masks only ever grow along K, so they are applied in place.
   __device__ __forceinline__ void mask_k_tail(int krem, int wave, int lane) {
 #pragma unroll
     for (int j = 0; j < IPW; ++j) {
       if constexpr (KMAJOR) {
-        uint32_t row = (wave * IPW + j) * 16 + (lane >> 2);
-        uint32_t c = (lane & 3) ^ swz_k(row);
+        uint32_t row = (wave * IPW + j) * 8 + (lane >> 3);
+        uint32_t c = (lane & 7) ^ swz_k(row);
         if ((int)c * 8 >= krem) voff[j] = OOB_OFFSET;
       } else {
         uint32_t krow = (wave * IPW + j) * KR + lane / CPR;
@@ -189,25 +196,30 @@ struct Operand {
     r[3] = 0x00020000;
     return r;
   }
-  // load j of this wave for the slab image at lds_img; M0 must hold lds_img + lds_w (dma_set_m0)
+  // load J of this wave; M0 must hold image + lds_w + (J / 4) * 4096 (dma_set_m0)
   template <int J>
   __device__ __forceinline__ void issue_one(i32x4 r) const {
-    dma16<J * 1024>(r, voff[J]);
+    dma16<(J & 3) * 1024>(r, voff[J]);
   }
   __device__ __forceinline__ void advance() { base += kadv; }
 };
 
-// Per-lane constants for reading MFMA operand fragments out of a slab image.  A fragment is the
+// Per-lane constants for reading MFMA operand fragments out of an image.  A fragment is the
 // 16 rows x 32 k operand of v_mfma_f32_16x16x32_bf16: lane l holds row (l & 15), k = 8*(l >> 4) .. +7.
 template <int ROWS, bool KMAJOR, int NT>
 struct FragReader {
   static constexpr int ROWB = ROWS * 2;
-  uint32_t lane_off[KMAJOR ? 1 : NT];
+  // LDS address of this lane's piece in image 0 of the operand's region: K-major, one per slab of the
+  // tile (fragment t is t * 2048 further); MN-major, one per fragment.  Image and fragment offsets are
+  // compile-time constants wherever possible so that they end up in the 16-bit offset field of ds_read.
+  uint32_t lane_off[KMAJOR ? 2 : NT];
 
-  __device__ __forceinline__ void init(int wrow0, int lane) {
+  __device__ __forceinline__ void init(uint32_t region, int wrow0, int lane) {
     if constexpr (KMAJOR) {
       const uint32_t row = lane & 15;
-      lane_off[0] = (uint32_t)(wrow0 + row) * 64 + ((((uint32_t)lane >> 4) ^ swz_k(row)) << 4);
+#pragma unroll
+      for (int s = 0; s < 2; ++s)
+        lane_off[s] = region + (uint32_t)(wrow0 + row) * 128 + (((4 * s + ((uint32_t)lane >> 4)) ^ swz_k(row)) << 4);
     } else {
       const uint32_t i = lane & 15, q = lane >> 4;
       const uint32_t tr_r = i >> 2, tr_c = i & 3;
@@ -215,36 +227,50 @@ struct FragReader {
 #pragma unroll
       for (int t = 0; t < NT; ++t) {
         uint32_t chunk = (uint32_t)(wrow0 >> 3) + 2 * t + (tr_c >> 1);
-        lane_off[t] = krow * ROWB + ((chunk ^ swz_mn(krow)) << 4) + ((tr_c & 1) << 3);
+        lane_off[t] = region + krow * ROWB + ((chunk ^ swz_mn(krow)) << 4) + ((tr_c & 1) << 3);
       }
     }
   }
-  // fragment t (16 rows, all 32 k) of the slab image at LDS address `img`
-  __device__ __forceinline__ bf16x8 read(uint32_t img, int t) const {
+  // MN-major: the two halves (k 0..3 and 4..7 of each lane's eight) of fragment t in the image at `img`
+  // (byte offset within the region)
+  __device__ __forceinline__ i16x4 read_half(uint32_t img, int t, int h) const {
+    return lds_read_tr16(lane_off[t] + img + h * 4 * ROWB);
+  }
+  // fragment t (16 rows) of slab `slab` (its parity picks the half of a K-major tile image)
+  __device__ __forceinline__ bf16x8 read(uint32_t img, int t, int slab) const {
     if constexpr (KMAJOR) {
-      return lds_read_b128(img + lane_off[0] + t * 1024);
+      return lds_read_b128(lane_off[slab & 1] + img + t * 2048);
     } else {
-      i16x4 lo = lds_read_tr16(img + lane_off[t]);
-      i16x4 hi = lds_read_tr16(img + lane_off[t] + 4 * ROWB);
-      i16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+      i16x8 v = __builtin_shufflevector(read_half(img, t, 0), read_half(img, t, 1), 0, 1, 2, 3, 4, 5, 6, 7);
       return __builtin_bit_cast(bf16x8, v);
     }
   }
 };
+__device__ __forceinline__ bf16x8 with_half(bf16x8 f, i16x4 h, int which) {
+  const i16x8 v = __builtin_bit_cast(i16x8, f);
+  const i16x8 w = __builtin_shufflevector(h, h, 0, 1, 2, 3, 0, 1, 2, 3);
+  const i16x8 r = which == 0 ? __builtin_shufflevector(w, v, 0, 1, 2, 3, 12, 13, 14, 15)
+                             : __builtin_shufflevector(v, w, 0, 1, 2, 3, 8, 9, 10, 11);
+  return __builtin_bit_cast(bf16x8, r);
+}
 
 // PROF adds s_memtime stamps around the two waits of the main loop and writes, per wave,
 // {total, waiting for own loads, waiting at the barrier, epilogue} shader-clock cycles to p.prof — the
 // per-phase cycle buffer idea of the reference's harness (cublass/matmul.cu:99-106,149-165).
-template <int BM, int BN, int WGM, int WGN, int NSLAB, bool AK, bool BK, bool PROF = false>
+template <int BM, int BN, int WGM, int WGN, bool AK, bool BK, bool PROF = false>
 __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
   constexpr int NW = WGM * WGN;
   constexpr int WTM = BM / WGM, WTN = BN / WGN;
   constexpr int TM = WTM / 16, TN = WTN / 16;
-  constexpr uint32_t A_BYTES = BM * KT * 2, B_BYTES = BN * KT * 2, SLAB = A_BYTES + B_BYTES;
   static_assert(WTM % 16 == 0 && WTN % 16 == 0, "wave tile must be a multiple of the 16x16 MFMA tile");
-  using OpA = Operand<BM, AK, NW>;
-  using OpB = Operand<BN, BK, NW>;
-  constexpr int LA = OpA::IPW, LB = OpB::IPW, LPS = LA + LB;  // this wave's loads per slab
+  static_assert(AK || BK, "at least one operand is K-major");
+  // images per operand: four 32-deep slabs if MN-major; 64-deep tiles if K-major, three of them next to
+  // an MN-major operand (160 KiB of LDS for a 256x256 tile), two if both operands are K-major
+  using OpA = Operand<BM, AK, NW, AK ? (BK ? 2 : 3) : 4>;
+  using OpB = Operand<BN, BK, NW, BK ? (AK ? 2 : 3) : 4>;
+  constexpr uint32_t A_BYTES = OpA::UNITS * OpA::IMG, LDS_BYTES = A_BYTES + OpB::UNITS * OpB::IMG;
+  constexpr int TU = (AK && BK) ? 2 : 3;  // images of a K-major operand
+  constexpr int IA = OpA::IPW, IB = OpB::IPW;  // this wave's loads per unit of A / of B
 
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   const uint32_t lds0 = (uint32_t)(uintptr_t)(NEOGEMM_AS3 char*)smem;
@@ -270,11 +296,12 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
     n0 = (rem / gsz) * BN;
   }
   const int kz = blockIdx.y;
-  const int k_begin = kz * p.ktiles_per_split * KT;
-  int k_end = k_begin + p.ktiles_per_split * KT;
+  const int k_begin = kz * p.ktiles_per_split * KTILE;
+  int k_end = k_begin + p.ktiles_per_split * KTILE;
   if (k_end > p.K) k_end = p.K;
-  const int nslab = (k_end - k_begin + KT - 1) / KT;
-  const int k_tail = (k_end - k_begin) - (nslab - 1) * KT;  // depth of the last slab, 1..KT
+  const int klen = k_end - k_begin;
+  const int ntile = (klen + KTILE - 1) / KTILE;
+  const int nslab = 2 * ntile;  // the last slab of a K-major tile may lie entirely past K: it is loaded as zeros
 
   unsigned long long t_start = 0, t_loads = 0, t_barrier = 0;
   if constexpr (PROF) t_start = __builtin_readcyclecounter();
@@ -285,8 +312,8 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
   opb.init(p.B, p.ldb, p.N, n0, k_begin, wave, lane);
   FragReader<BM, AK, TM> fa;
   FragReader<BN, BK, TN> fb;
-  fa.init(wm * WTM, lane);
-  fb.init(wn * WTN, lane);
+  fa.init(lds0, wm * WTM, lane);
+  fb.init(lds0 + A_BYTES, wn * WTN, lane);
 
   f32x4 acc[TM][TN];
 #pragma unroll
@@ -300,75 +327,153 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
   constexpr int HM = TM / 2;
   bf16x8 af[TM], bfr[TN];  // one copy of each fragment; refreshed in place as soon as it is dead
 
-  auto img_of = [&](int slab) -> uint32_t { return lds0 + (uint32_t)(slab % NSLAB) * SLAB; };
+  // LDS image that holds slab j of an operand
+  // (byte offset within the operand's region)
+  auto img_a = [&](int j) -> uint32_t { return (AK ? ((uint32_t)(j >> 1) % TU) : ((uint32_t)j & 3u)) * OpA::IMG; };
+  auto img_b = [&](int j) -> uint32_t { return (BK ? ((uint32_t)(j >> 1) % TU) : ((uint32_t)j & 3u)) * OpB::IMG; };
+
+  // Which of this wave's loads go under which half-step.  The schedule has a period of two slabs
+  // (four half-steps P0..P3, starting after the sync that follows an odd slab's first half):
+  //   a K-major operand loads one 64-deep tile per period, in P0 and P1 (both K-major: over P0..P2);
+  //   an MN-major operand loads one slab in P2 and one in P3.
+  // Segment = loads [lo, hi) of operand A (op 1) or B (op 2); a half-step carries up to two segments.
+  struct Seg { int op, lo, hi; };
+  auto plan = [](int phase, int which) constexpr -> Seg {
+    if (AK && BK) {
+      // 16 (IA + IB) loads over P0, P1, P2
+      const int tot = IA + IB, c0 = (tot + 2) / 3, c1 = (tot - c0 + 1) / 2;  // P0: [0,c0) P1: [c0,c0+c1) P2: rest
+      const int lo = phase == 0 ? 0 : (phase == 1 ? c0 : (phase == 2 ? c0 + c1 : tot));
+      const int hi = phase == 0 ? c0 : (phase == 1 ? c0 + c1 : tot);
+      // split [lo,hi) of the concatenation A[0,IA) B[0,IB) into the A part (which 0) and the B part (which 1)
+      if (which == 0) return Seg{1, lo < IA ? lo : IA, hi < IA ? hi : IA};
+      return Seg{2, (lo > IA ? lo : IA) - IA, (hi > IA ? hi : IA) - IA};
+    } else if (AK) {
+      if (which == 1) return Seg{0, 0, 0};
+      if (phase == 0) return Seg{1, 0, IA / 2};
+      if (phase == 1) return Seg{1, IA / 2, IA};
+      return Seg{2, 0, IB};
+    } else {
+      if (which == 1) return Seg{0, 0, 0};
+      if (phase == 0) return Seg{2, 0, IB / 2};
+      if (phase == 1) return Seg{2, IB / 2, IB};
+      return Seg{1, 0, IA};
+    }
+  };
 
   // Half a slab step: the MFMAs of fragment rows [HALF*HM, HALF*HM + HM) against every B fragment,
-  // column by column, with the LDS reads that refresh dead fragments and (DMA) this wave's loads of
-  // one operand of a later slab, one load after every few columns.  The wave issues in order, and
-  // whatever sits between two MFMAs beyond the 16 cycles the first one occupies the pipe is lost, so
-  // memory instructions are never issued in bursts.
-  //   HALF 0 reads the second-half A fragments of the slab being computed (image img_rd).
-  //   HALF 1 reads, from the next slab's image img_rd, the first-half A fragments and, after the last
-  //   MFMA that uses it, each B fragment.
-  auto half_step = [&](auto half, auto do_read, uint32_t img_rd, auto do_dma, uint32_t img_dma) {
-    constexpr int HALF = decltype(half)::value;
-    constexpr bool READ = decltype(do_read)::value, DMA = decltype(do_dma)::value;
-    constexpr int NL = DMA ? (HALF == 1 ? LA : LB) : 0;  // A part under half 1, B part under the next half 0
-    constexpr int APC = (HM + TN - 1) / TN;               // A fragments refreshed per column
-    i32x4 rs;
-    if constexpr (DMA) {
-      rs = HALF == 1 ? opa.rsrc() : opb.rsrc();
-      dma_set_m0(HALF == 1 ? img_dma + opa.lds_w : img_dma + A_BYTES + opb.lds_w);
+  // column by column, with the LDS reads that refresh dead fragments and, when PHASE >= 0, the loads
+  // the schedule puts under this half-step.  The wave issues in order, about one instruction every four
+  // cycles, and whatever sits between two MFMAs beyond the 16 cycles the first one occupies the pipe is
+  // lost: the memory instructions are dealt out one per gap between MFMAs as far as the gaps go.
+  //   HALF 0 reads the second-half A fragments of the slab being computed (slab_rd).
+  //   HALF 1 reads, from the next slab slab_rd, the first-half A fragments and, after the last MFMA
+  //   that uses it, each B fragment.  An MN-major B fragment takes two reads: the second one goes
+  //   after the first MFMA of the next column; that of the last column is left to the HALF 0 step that
+  //   follows (PEND), which reads from the same slab.
+  // ia / ib: image (offset in the operand's region) the fragments are read from;
+  // dst_a / dst_b: LDS address of the image the A / B loads of this half-step go to.
+  auto half_step = [&](auto half, auto do_read, auto pend, int slab_rd, uint32_t ia, uint32_t ib, auto phase,
+                       uint32_t dst_a, uint32_t dst_b) {
+    constexpr int HALF = decltype(half)::value, PHASE = decltype(phase)::value;
+    constexpr bool READ = decltype(do_read)::value, PEND = decltype(pend)::value;
+    constexpr Seg s0 = PHASE >= 0 ? plan(PHASE, 0) : Seg{0, 0, 0}, s1 = PHASE >= 0 ? plan(PHASE, 1) : Seg{0, 0, 0};
+    constexpr int n0l = s0.hi - s0.lo, n1l = s1.hi - s1.lo, NL = n0l + n1l;
+    constexpr int APC = (HM + TN - 1) / TN;  // A fragments refreshed per column
+    constexpr bool SPLIT_B = !BK && HM >= 2;  // B fragment reads in two halves, one gap apart
+    i32x4 ra, rb;
+    if constexpr (NL > 0) {
+      ra = opa.rsrc();
+      rb = opb.rsrc();
     }
+    // the l-th load of this half-step
+    auto issue = [&](auto lc) {
+      constexpr int l = decltype(lc)::value;
+      constexpr Seg sg = l < n0l ? s0 : s1;
+      constexpr int J = l < n0l ? s0.lo + l : s1.lo + (l - n0l);
+      constexpr bool first = (l == 0) || (l == n0l) || (J % 4 == 0);
+      if constexpr (sg.op == 1) {
+        if constexpr (first) dma_set_m0(dst_a + opa.lds_w + (J / 4) * 4096);
+        opa.template issue_one<J>(ra);
+      } else {
+        if constexpr (first) dma_set_m0(dst_b + opb.lds_w + (J / 4) * 4096);
+        opb.template issue_one<J>(rb);
+      }
+    };
     static_for<TN>([&](auto cc) {
       constexpr int c = decltype(cc)::value;
       constexpr int a_lo = c * APC < HM ? c * APC : HM, a_hi = (c + 1) * APC < HM ? (c + 1) * APC : HM;
-      constexpr int l_lo = c * NL / TN, l_hi = (c + 1) * NL / TN;  // loads: NL of them spread over the TN columns
-      // Column c: HM MFMAs.  At most one memory instruction goes between two MFMAs: the A refreshes
-      // after the first MFMA, the direct-to-LDS load after the second, the B refresh after the last
-      // (which is the last reader of bfr[c]).
+      constexpr int l_lo = c * NL / TN, l_hi = (c + 1) * NL / TN;  // loads spread over the TN columns
+      // memory instructions of this column in order: [second half of the previous column's B fragment]
+      // [A fragments] [loads]; the k-th goes into gap min(k, HM-1); the B read of this column always
+      // follows the column's last MFMA
+      constexpr int cprev = c == 0 ? TN - 1 : c - 1;
+      constexpr bool bhi = SPLIT_B && ((HALF == 1 && READ && c > 0) || (HALF == 0 && PEND && c == 0));
+      constexpr int nA = READ ? a_hi - a_lo : 0, nLd = l_hi - l_lo;
       static_for<HM>([&](auto ic) {
         constexpr int ii = decltype(ic)::value;
         constexpr int i = HALF * HM + ii;
         // B fragment first: D rows index n, D columns index m, so a lane ends up with 4
-        // consecutive n of one output row (an 8-byte store) instead of 4 rows of one column.
+        // consecutive n of one output row (an 8-byte piece) instead of 4 rows of one column.
         mfma_16x16x32(acc[i][c], bfr[c], af[i]);
-        if constexpr (READ && ii == 0) {
-#pragma unroll
-          for (int f = a_lo; f < a_hi; ++f) {
-            if constexpr (HALF == 0) af[HM + f] = fa.read(img_rd, HM + f);
-            else af[f] = fa.read(img_rd, f);
+        static_for<(bhi ? 1 : 0) + nA + nLd>([&](auto kc) {
+          constexpr int k = decltype(kc)::value;
+          if constexpr ((k < HM - 1 ? k : HM - 1) == ii) {
+            if constexpr (bhi && k == 0) {
+              bfr[cprev] = with_half(bfr[cprev], fb.read_half(ib, cprev, 1), 1);
+            } else if constexpr (k - (bhi ? 1 : 0) < nA) {
+              constexpr int f = a_lo + k - (bhi ? 1 : 0);
+              if constexpr (HALF == 0) af[HM + f] = fa.read(ia, HM + f, slab_rd);
+              else af[f] = fa.read(ia, f, slab_rd);
+            } else {
+              issue(std::integral_constant<int, l_lo + k - (bhi ? 1 : 0) - nA>{});
+            }
           }
-        }
-        if constexpr (ii == (HM > 1 ? 1 : 0) && l_hi > l_lo) {
-          static_for<l_hi - l_lo>([&](auto lc) {
-            constexpr int l = l_lo + decltype(lc)::value;
-            if constexpr (HALF == 1) opa.template issue_one<l>(rs);
-            else opb.template issue_one<l>(rs);
-          });
-        }
+        });
       });
-      if constexpr (READ && HALF == 1) bfr[c] = fb.read(img_rd + A_BYTES, c);
+      if constexpr (READ && HALF == 1) {
+        if constexpr (SPLIT_B) {
+          bfr[c] = with_half(bfr[c], fb.read_half(ib, c, 0), 0);
+          if constexpr (c == TN - 1 && !PEND) bfr[c] = with_half(bfr[c], fb.read_half(ib, c, 1), 1);
+        } else {
+          bfr[c] = fb.read(ib, c, slab_rd);
+        }
+      }
     });
-    if constexpr (DMA) {
-      if constexpr (HALF == 1) opa.advance();
-      else opb.advance();
+    // the unit of an operand is complete once its last load is out: move its resource along K
+    if constexpr (NL > 0) {
+      if constexpr ((s0.op == 1 && s0.hi == IA && n0l > 0) || (s1.op == 1 && s1.hi == IA && n1l > 0)) opa.advance();
+      if constexpr ((s0.op == 2 && s0.hi == IB && n0l > 0) || (s1.op == 2 && s1.hi == IB && n1l > 0)) opb.advance();
     }
   };
 
-  auto load_slab_burst = [&](int j) {
-    if (j == nslab - 1 && k_tail != KT) {
-      opa.mask_k_tail(k_tail, wave, lane);
-      opb.mask_k_tail(k_tail, wave, lane);
-    }
-    const i32x4 ra = opa.rsrc(), rb = opb.rsrc();
-    dma_set_m0(img_of(j) + opa.lds_w);
-    static_for<LA>([&](auto lc) { opa.template issue_one<decltype(lc)::value>(ra); });
-    dma_set_m0(img_of(j) + A_BYTES + opb.lds_w);
-    static_for<LB>([&](auto lc) { opb.template issue_one<decltype(lc)::value>(rb); });
+  // All loads of one unit of an operand in a burst (prologue and tail).  `unit` counts tiles for a
+  // K-major operand and slabs for an MN-major one; the last units get their K tail masked.
+  auto burst_a = [&](int unit) {
+    const int krem = klen - unit * OpA::UNIT_K;
+    if (krem < OpA::UNIT_K) opa.mask_k_tail(krem, wave, lane);
+    const i32x4 r = opa.rsrc();
+    const uint32_t dst = lds0 + (uint32_t)(unit % OpA::UNITS) * OpA::IMG + opa.lds_w;
+    static_for<IA>([&](auto lc) {
+      constexpr int J = decltype(lc)::value;
+      if constexpr (J % 4 == 0) dma_set_m0(dst + (J / 4) * 4096);
+      opa.template issue_one<J>(r);
+    });
     opa.advance();
+  };
+  auto burst_b = [&](int unit) {
+    const int krem = klen - unit * OpB::UNIT_K;
+    if (krem < OpB::UNIT_K) opb.mask_k_tail(krem, wave, lane);
+    const i32x4 r = opb.rsrc();
+    const uint32_t dst = lds0 + A_BYTES + (uint32_t)(unit % OpB::UNITS) * OpB::IMG + opb.lds_w;
+    static_for<IB>([&](auto lc) {
+      constexpr int J = decltype(lc)::value;
+      if constexpr (J % 4 == 0) dma_set_m0(dst + (J / 4) * 4096);
+      opb.template issue_one<J>(r);
+    });
     opb.advance();
   };
+  const int nunit_a = AK ? ntile : nslab, nunit_b = BK ? ntile : nslab;
+
   // Wait until this wave's loads of the slab about to be read have landed (all but the `keep` most
   // recent loads), and its own LDS reads are done; then meet the other waves.
   auto sync = [&](auto keep) {
@@ -396,55 +501,82 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
   using F = std::false_type;
   using H0 = std::integral_constant<int, 0>;
   using H1 = std::integral_constant<int, 1>;
+  using NoLoads = std::integral_constant<int, -1>;
 
-  // Ring of NSLAB slab images; slab j lives in image j % NSLAB.  The work on slab j is
-  //   half 0   MFMAs of the first-half rows; reads the second-half A fragments of slab j;
-  //            streams the B part of slab j+3 into image (j+3)%4
-  //   sync     every wave has all fragments of slab j in registers (image j%4 may be overwritten)
-  //            and slab j+1 has landed for all of them
-  //   half 1   MFMAs of the second-half rows; reads from slab j+1 the first-half A fragments and
-  //            each B fragment right after its last use; streams the A part of slab j+4 into image j%4
-  // so a load has at least two slab-times to land, loads leave the wave one at a time, and only one
-  // copy of each fragment is held in registers.  The loop below is rotated: one iteration is
-  // sync, half 1 of slab j, half 0 of slab j+1.
-  {
-    const int npre = nslab < NSLAB ? nslab : NSLAB;
-    for (int jj = 0; jj < npre; ++jj) load_slab_burst(jj);
-    // slab 0 landed: everything but the later slabs' loads
-    if (npre == 4) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * LPS) : "memory");
-    else if (npre == 3) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * LPS) : "memory");
-    else if (npre == 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LPS) : "memory");
-    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-  }
-#pragma unroll
-  for (int t = 0; t < HM; ++t) af[t] = fa.read(img_of(0), t);
-#pragma unroll
-  for (int t = 0; t < TN; ++t) bfr[t] = fb.read(img_of(0) + A_BYTES, t);
-  half_step(H0{}, T{}, img_of(0), F{}, 0);
+  // One iteration j of the rotated loop is: sync, second half of slab j, first half of slab j+1.
+  // After the sync every wave holds all fragments of slab j in registers and slab j+1 has landed, so
+  //   an MN-major slab image j & 3 is dead and takes slab j+4;
+  //   for odd j the K-major tile image (j >> 1) % TU is dead and takes tile (j >> 1) + TU.
+  // Steady state, period t (iterations j = 2t+1 and 2t+2), what is issued and what each sync keeps in
+  // flight (loads complete in issue order):
+  //   one K-major operand X (three images), the other Y MN-major:
+  //     P0 = second half of slab 2t+1: first half of X tile t+3      P1 = first half of slab 2t+2: the rest
+  //     P2 = second half of slab 2t+2: Y slab 2t+5                   P3 = first half of slab 2t+3: Y slab 2t+6
+  //     the sync before P0 needs X tile t+1 and Y slab 2t+2: all but the loads of the period before
+  //     the sync before P2 needs Y slab 2t+3: all but Y slab 2t+4 and X tile t+3
+  //   both K-major (two images): tile t+2 of both over P0..P2; only the sync before P0 is needed, and
+  //   it needs everything
+  constexpr int KEEP_ODD = (AK && BK) ? 0 : (IA + IB + (AK ? IB : IA));
+  constexpr int KEEP_EVEN = (AK && BK) ? -1 : IA + IB;
 
-  int j = 0;
-  // steady: slab j+4 exists and is not the last one (the last may need its K tail masked)
-  for (; j + (NSLAB - 1) + NSLAB < nslab - 1; j += NSLAB) {
+  // prologue: two tiles / four slabs of each operand, all landed
+  for (int u = 0; u < OpA::UNITS && u < nunit_a; ++u) burst_a(u);
+  for (int u = 0; u < OpB::UNITS && u < nunit_b; ++u) burst_b(u);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
 #pragma unroll
-    for (int u = 0; u < NSLAB; ++u) {
-      const uint32_t img_free = lds0 + u * SLAB, img_next = lds0 + ((u + 1) % NSLAB) * SLAB;
-      sync(std::integral_constant<int, (NSLAB - 2) * LPS>{});
-      half_step(H1{}, T{}, img_next, T{}, img_free);
-      half_step(H0{}, T{}, img_next, T{}, img_free);
+  for (int t = 0; t < HM; ++t) af[t] = fa.read(img_a(0), t, 0);
+#pragma unroll
+  for (int t = 0; t < TN; ++t) bfr[t] = fb.read(img_b(0), t, 0);
+  half_step(H0{}, T{}, F{}, 0, img_a(0), img_b(0), NoLoads{}, 0, 0);
+
+  // iteration with loads in a burst and full waits: j = 0, and the tail
+  auto slow_iteration = [&](int j) {
+    sync(std::integral_constant<int, 0>{});
+    if constexpr (!AK) { if (j + 4 < nslab) burst_a(j + 4); }
+    if constexpr (!BK) { if (j + 4 < nslab) burst_b(j + 4); }
+    if (j & 1) {
+      if constexpr (AK) { if ((j >> 1) + TU < ntile) burst_a((j >> 1) + TU); }
+      if constexpr (BK) { if ((j >> 1) + TU < ntile) burst_b((j >> 1) + TU); }
+    }
+    half_step(H1{}, T{}, T{}, j + 1, img_a(j + 1), img_b(j + 1), NoLoads{}, 0, 0);
+    half_step(H0{}, T{}, T{}, j + 1, img_a(j + 1), img_b(j + 1), NoLoads{}, 0, 0);
+  };
+  slow_iteration(0);
+
+  int j = 1;
+  // steady: two periods per trip (the MN-major slab images repeat every four slabs, the K-major
+  // tile images rotate at run time); every unit loaded here exists and is full
+  uint32_t x_ld = 0, x_rd = 1;  // tile image that takes tile t+TU (= image of tile t) / that holds tile t+1
+  for (; (j >> 1) + 4 < ntile - 1; j += 4) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      // period t = (j >> 1) + u, t & 1 == u since j == 1 (mod 4)
+      const int jo = j + 2 * u;  // the odd slab 2t+1
+      // slab images (2t+1) & 3 and (2t+2) & 3 take slabs 2t+5 and 2t+6; slabs 2t+2, 2t+3 are read
+      const uint32_t da0 = lds0 + (AK ? x_ld : (uint32_t)((2 * u + 1) & 3)) * OpA::IMG;
+      const uint32_t da1 = lds0 + (AK ? x_ld : (uint32_t)((2 * u + 2) & 3)) * OpA::IMG;
+      const uint32_t db0 = lds0 + A_BYTES + (BK ? x_ld : (uint32_t)((2 * u + 1) & 3)) * OpB::IMG;
+      const uint32_t db1 = lds0 + A_BYTES + (BK ? x_ld : (uint32_t)((2 * u + 2) & 3)) * OpB::IMG;
+      const uint32_t ra0 = (AK ? x_rd : (uint32_t)((2 * u + 2) & 3)) * OpA::IMG;
+      const uint32_t ra1 = (AK ? x_rd : (uint32_t)((2 * u + 3) & 3)) * OpA::IMG;
+      const uint32_t rb0 = (BK ? x_rd : (uint32_t)((2 * u + 2) & 3)) * OpB::IMG;
+      const uint32_t rb1 = (BK ? x_rd : (uint32_t)((2 * u + 3) & 3)) * OpB::IMG;
+      sync(std::integral_constant<int, KEEP_ODD>{});
+      half_step(H1{}, T{}, T{}, jo + 1, ra0, rb0, std::integral_constant<int, 0>{}, da0, db0);
+      half_step(H0{}, T{}, T{}, jo + 1, ra0, rb0, std::integral_constant<int, 1>{}, da0, db0);
+      if constexpr (KEEP_EVEN >= 0) sync(std::integral_constant<int, KEEP_EVEN>{});
+      half_step(H1{}, T{}, T{}, jo + 2, ra1, rb1, std::integral_constant<int, 2>{}, da0, db0);
+      half_step(H0{}, T{}, T{}, jo + 2, ra1, rb1, std::integral_constant<int, 3>{}, da1, db1);
+      x_ld = x_rd;
+      x_rd = x_rd + 1 == TU ? 0 : x_rd + 1;
     }
   }
-  // tail: runtime slab indices, loads in a burst, conservative waits
-  for (; j + 1 < nslab; ++j) {
-    sync(std::integral_constant<int, 0>{});
-    if (j + NSLAB < nslab) load_slab_burst(j + NSLAB);
-    half_step(H1{}, T{}, img_of(j + 1), F{}, 0);
-    half_step(H0{}, T{}, img_of(j + 1), F{}, 0);
-  }
+  for (; j + 1 < nslab; ++j) slow_iteration(j);
   // second half of the last slab: its fragments are in registers or on their way from LDS; every
-  // load was waited for by the last sync (or the prologue when there is one slab)
-  half_step(H1{}, F{}, 0, F{}, 0);
+  // load was waited for by the last sync
+  half_step(H1{}, F{}, F{}, 0, 0, 0, NoLoads{}, 0, 0);
 
   // The last MFMAs must have left the pipe before their accumulators are read, and the compiler,
   // which sees neither MFMAs nor hazard here, inserts nothing.  Volatile asm statements keep their
@@ -465,7 +597,7 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
   // so that neither the 8-byte writes (16 rows per instruction) nor the 16-byte reads collide on banks.
   constexpr int CH = WTN / 8;        // 16-byte chunks per staged row
   constexpr int RPI = 64 / CH;       // rows one store instruction covers
-  constexpr bool CAN_STAGE = (size_t)BM * BN * 2 <= (size_t)NSLAB * SLAB && CH >= 4 && CH <= 64;
+  constexpr bool CAN_STAGE = (size_t)BM * BN * 2 <= (size_t)LDS_BYTES && CH >= 4 && CH <= 64;
   const bool stage = CAN_STAGE && p.ksplit == 1 && (((uintptr_t)p.C | (uintptr_t)(p.ldc * 2)) & 15) == 0;
   if (stage) {
     if constexpr (CAN_STAGE) {
@@ -624,9 +756,10 @@ static const VariantInfo kVariants[NEOGEMM_VARIANT_COUNT] = {
     {0, 0, 0}, {16, 16, 4}, {256, 256, 8}, {256, 256, 4}, {128, 128, 4}, {256, 128, 8}, {128, 256, 8}, {64, 128, 4}, {128, 128, 4},
 };
 
-template <int BM, int BN, int WGM, int WGN, int NSLAB>
+template <int BM, int BN, int WGM, int WGN>
 static hipError_t launch_tile(const TileArgs& a, bool ak, bool bk, hipStream_t st) {
-  constexpr size_t lds = (size_t)NSLAB * (BM + BN) * KT * 2;
+  // four 32-deep images of an MN-major operand; three 64-deep ones of a K-major operand next to it, two if both are K-major
+  const size_t lds = (ak && bk) ? (size_t)(BM + BN) * 256 : (size_t)(ak ? BM : BN) * 384 + (size_t)(ak ? BN : BM) * 256;
   dim3 grid(a.ntm * a.ntn, a.ksplit), block(WGM * WGN * 64);
   auto go = [&](auto kern) -> hipError_t {
     static bool attr_done = false;  // per instantiation
@@ -640,17 +773,17 @@ static hipError_t launch_tile(const TileArgs& a, bool ak, bool bk, hipStream_t s
   };
   if (a.prof) {
     if constexpr (BM == 256 && BN == 256) {
-      if (ak && bk) return go(gemm_tile_kernel<BM, BN, WGM, WGN, NSLAB, true, true, true>);
-      if (ak && !bk) return go(gemm_tile_kernel<BM, BN, WGM, WGN, NSLAB, true, false, true>);
+      if (ak && bk) return go(gemm_tile_kernel<BM, BN, WGM, WGN, true, true, true>);
+      if (ak && !bk) return go(gemm_tile_kernel<BM, BN, WGM, WGN, true, false, true>);
     }
     return hipErrorInvalidValue;
   }
-  if (ak && bk) return go(gemm_tile_kernel<BM, BN, WGM, WGN, NSLAB, true, true>);
+  if (ak && bk) return go(gemm_tile_kernel<BM, BN, WGM, WGN, true, true>);
   if (ak && !bk) {
-    if constexpr (BN >= 128) return go(gemm_tile_kernel<BM, BN, WGM, WGN, NSLAB, true, false>);
+    if constexpr (BN >= 128) return go(gemm_tile_kernel<BM, BN, WGM, WGN, true, false>);
   }
   if (!ak && bk) {
-    if constexpr (BM >= 128) return go(gemm_tile_kernel<BM, BN, WGM, WGN, NSLAB, false, true>);
+    if constexpr (BM >= 128) return go(gemm_tile_kernel<BM, BN, WGM, WGN, false, true>);
   }
   return hipErrorInvalidValue;
 }
@@ -672,7 +805,7 @@ static void plan(int64_t M, int64_t N, int64_t K, bool aligned, int c_layout, in
     return;
   }
   const int64_t rows = c_layout == NEOGEMM_C_ROW ? M : N, cols = c_layout == NEOGEMM_C_ROW ? N : M;
-  const int64_t ktiles = ceil_div(K, KT);
+  const int64_t ktiles = ceil_div(K, KTILE);
   int v, slots;  // slots: workgroups of this variant the 256 CUs hold at once (LDS-limited)
   if ((int64_t)ceil_div(rows, 256) * ceil_div(cols, 256) >= 64 && rows > 128 && cols > 128) {
     // One wave per SIMD with a 128x128 wave tile reads the least LDS per flop.
@@ -693,9 +826,9 @@ static void plan(int64_t M, int64_t N, int64_t K, bool aligned, int c_layout, in
   int s = 1;
   if (tiles * 4 < slots * 3) {
     // not enough tiles to fill the chip: split K so that one round of workgroups covers the CUs,
-    // keeping >= 8 slabs per split so the pipeline has something to overlap
+    // keeping >= 4 K tiles (256 deep) per split so the pipeline has something to overlap
     int64_t want = slots / tiles;
-    int64_t maxs = ktiles / 8 > 0 ? ktiles / 8 : 1;
+    int64_t maxs = ktiles / 4 > 0 ? ktiles / 4 : 1;
     s = (int)(want < maxs ? want : maxs);
     if (s < 1) s = 1;
     if (s > 64) s = 64;
@@ -763,10 +896,10 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
   const VariantInfo& vi = kVariants[v];
   // What the tile kernels assume about an operand (see Operand::init): an MN-major tile needs >= 128
   // rows for its swizzle, ld >= tile rows and a row count that is a multiple of 8 (16-byte chunks must
-  // not straddle the matrix edge), a K-major one ld >= 32, so that the per-lane offsets, which are
+  // not straddle the matrix edge), a K-major one ld >= 64, so that the per-lane offsets, which are
   // biased by the instruction offsets of the loads, stay non-negative.
-  const bool fits = (ak ? a.lda >= 32 : (vi.bm >= 128 && a.lda >= vi.bm && (a.M & 7) == 0)) &&
-                    (bk ? a.ldb >= 32 : (vi.bn >= 128 && a.ldb >= vi.bn && (a.N & 7) == 0));
+  const bool fits = (ak ? a.lda >= 64 : (vi.bm >= 128 && a.lda >= vi.bm && (a.M & 7) == 0)) &&
+                    (bk ? a.ldb >= 64 : (vi.bn >= 128 && a.ldb >= vi.bn && (a.N & 7) == 0));
   if (!fits) {
     if (variant != NEOGEMM_VARIANT_AUTO) return NEOGEMM_ERR_UNSUPPORTED;
     // the planned tile is too wide for an MN-major operand: the 128x128 tile needs the least, then generic
@@ -782,7 +915,7 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
   a.ntn = ceil_div(a.N, vi.bn);
   if ((int64_t)a.ntm * a.ntn > 0x7fffffff) return NEOGEMM_ERR_UNSUPPORTED;
   a.group_m = group_m > 0 ? group_m : 8;
-  const int ktiles = ceil_div(K, KT);
+  const int ktiles = ceil_div(K, KTILE);
   if (s > ktiles) s = ktiles;
   a.ktiles_per_split = ceil_div(ktiles, s);
   a.ksplit = ceil_div(ktiles, a.ktiles_per_split);  // no empty split
@@ -798,13 +931,13 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
 
   hipError_t e;
   switch (v) {
-    case NEOGEMM_VARIANT_T256x256_W8: e = launch_tile<256, 256, 2, 4, 4>(a, ak, bk, st); break;
-    case NEOGEMM_VARIANT_T256x256_W4: e = launch_tile<256, 256, 2, 2, 4>(a, ak, bk, st); break;
-    case NEOGEMM_VARIANT_T128x128_W4: e = launch_tile<128, 128, 2, 2, 4>(a, ak, bk, st); break;
-    case NEOGEMM_VARIANT_T256x128_W8: e = launch_tile<256, 128, 4, 2, 4>(a, ak, bk, st); break;
-    case NEOGEMM_VARIANT_T128x256_W8: e = launch_tile<128, 256, 2, 4, 4>(a, ak, bk, st); break;
-    case NEOGEMM_VARIANT_T64x128_W4: e = launch_tile<64, 128, 1, 4, 6>(a, ak, bk, st); break;
-    case NEOGEMM_VARIANT_T128x128_W4S: e = launch_tile<128, 128, 1, 4, 5>(a, ak, bk, st); break;
+    case NEOGEMM_VARIANT_T256x256_W8: e = launch_tile<256, 256, 2, 4>(a, ak, bk, st); break;
+    case NEOGEMM_VARIANT_T256x256_W4: e = launch_tile<256, 256, 2, 2>(a, ak, bk, st); break;
+    case NEOGEMM_VARIANT_T128x128_W4: e = launch_tile<128, 128, 2, 2>(a, ak, bk, st); break;
+    case NEOGEMM_VARIANT_T256x128_W8: e = launch_tile<256, 128, 4, 2>(a, ak, bk, st); break;
+    case NEOGEMM_VARIANT_T128x256_W8: e = launch_tile<128, 256, 2, 4>(a, ak, bk, st); break;
+    case NEOGEMM_VARIANT_T64x128_W4: e = launch_tile<64, 128, 1, 4>(a, ak, bk, st); break;
+    case NEOGEMM_VARIANT_T128x128_W4S: e = launch_tile<128, 128, 1, 4>(a, ak, bk, st); break;
     default: return NEOGEMM_ERR_BAD_ARG;
   }
   if (e != hipSuccess) {
