@@ -236,7 +236,17 @@ struct FragReader {
   __device__ __forceinline__ i16x4 read_half(uint32_t img, int t, int h) const {
     return lds_read_tr16(lane_off[t] + img + h * 4 * ROWB);
   }
-  // fragment t (16 rows) of slab `slab` (its parity picks the half of a K-major tile image)
+  // K-major: this lane's address for slab `slab` (its parity picks the half of the tile image) in
+  // the image at `img`.  When img is not a compile-time constant the sum is pinned in a VGPR, so that
+  // the fragment offsets t * 2048 go into the offset field of the reads instead of being added, one
+  // scalar and one vector instruction per read, to the image offset first.
+  __device__ __forceinline__ uint32_t base(uint32_t img, int slab) const {
+    uint32_t b = lane_off[slab & 1] + img;
+    if (!__builtin_constant_p(img)) asm volatile("" : "+v"(b));
+    return b;
+  }
+  __device__ __forceinline__ bf16x8 read_at(uint32_t b, int t) const { return lds_read_b128(b + t * 2048); }
+  // fragment t (16 rows) of slab `slab`
   __device__ __forceinline__ bf16x8 read(uint32_t img, int t, int slab) const {
     if constexpr (KMAJOR) {
       return lds_read_b128(lane_off[slab & 1] + img + t * 2048);
@@ -264,12 +274,11 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
   constexpr int TM = WTM / 16, TN = WTN / 16;
   static_assert(WTM % 16 == 0 && WTN % 16 == 0, "wave tile must be a multiple of the 16x16 MFMA tile");
   static_assert(AK || BK, "at least one operand is K-major");
-  // images per operand: four 32-deep slabs if MN-major; 64-deep tiles if K-major, three of them next to
-  // an MN-major operand (160 KiB of LDS for a 256x256 tile), two if both operands are K-major
-  using OpA = Operand<BM, AK, NW, AK ? (BK ? 2 : 3) : 4>;
+  // images per operand: four 32-deep slabs if MN-major; three 64-deep tiles if K-major, except that
+  // B gets by with two when both are K-major (160 KiB of LDS for a 256x256 tile either way)
+  using OpA = Operand<BM, AK, NW, AK ? 3 : 4>;
   using OpB = Operand<BN, BK, NW, BK ? (AK ? 2 : 3) : 4>;
   constexpr uint32_t A_BYTES = OpA::UNITS * OpA::IMG, LDS_BYTES = A_BYTES + OpB::UNITS * OpB::IMG;
-  constexpr int TU = (AK && BK) ? 2 : 3;  // images of a K-major operand
   constexpr int IA = OpA::IPW, IB = OpB::IPW;  // this wave's loads per unit of A / of B
 
   extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -323,30 +332,27 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
 #pragma unroll
       for (int v = 0; v < 4; ++v) acc[i][j][v] = 0.f;
 
-  static_assert(TM % 2 == 0, "the wave tile is processed in two halves of TM/2 fragment rows");
-  constexpr int HM = TM / 2;
-  bf16x8 af[TM], bfr[TN];  // one copy of each fragment; refreshed in place as soon as it is dead
+  // Two copies of every fragment: slab j is computed from copy j & 1 while the fragments of slab j+1
+  // are read into the other one.  The accumulators live in the 256 AGPRs, so the VGPRs have room.
+  bf16x8 af[2][TM] = {}, bfr[2][TN] = {};
 
   // LDS image that holds slab j of an operand
   // (byte offset within the operand's region)
-  auto img_a = [&](int j) -> uint32_t { return (AK ? ((uint32_t)(j >> 1) % TU) : ((uint32_t)j & 3u)) * OpA::IMG; };
-  auto img_b = [&](int j) -> uint32_t { return (BK ? ((uint32_t)(j >> 1) % TU) : ((uint32_t)j & 3u)) * OpB::IMG; };
+  auto img_a = [&](int j) -> uint32_t { return ((uint32_t)(AK ? j >> 1 : j) % OpA::UNITS) * OpA::IMG; };
+  auto img_b = [&](int j) -> uint32_t { return ((uint32_t)(BK ? j >> 1 : j) % OpB::UNITS) * OpB::IMG; };
 
-  // Which of this wave's loads go under which half-step.  The schedule has a period of two slabs
-  // (four half-steps P0..P3, starting after the sync that follows an odd slab's first half):
-  //   a K-major operand loads one 64-deep tile per period, in P0 and P1 (both K-major: over P0..P2);
-  //   an MN-major operand loads one slab in P2 and one in P3.
-  // Segment = loads [lo, hi) of operand A (op 1) or B (op 2); a half-step carries up to two segments.
+  // Which of this wave's loads go under which half of a slab step.  The schedule has a period of two
+  // slabs (four halves P0..P3, starting with an odd slab):
+  //   next to an MN-major operand, a K-major one loads a 64-deep tile in P0 and P1, the MN-major one a
+  //   slab in P2 and one in P3; if both are K-major, B loads its tile in P0 and A over P1..P3.
+  // Segment = loads [lo, hi) of operand A (op 1) or B (op 2); a half carries up to two segments.
   struct Seg { int op, lo, hi; };
   auto plan = [](int phase, int which) constexpr -> Seg {
     if (AK && BK) {
-      // 16 (IA + IB) loads over P0, P1, P2
-      const int tot = IA + IB, c0 = (tot + 2) / 3, c1 = (tot - c0 + 1) / 2;  // P0: [0,c0) P1: [c0,c0+c1) P2: rest
-      const int lo = phase == 0 ? 0 : (phase == 1 ? c0 : (phase == 2 ? c0 + c1 : tot));
-      const int hi = phase == 0 ? c0 : (phase == 1 ? c0 + c1 : tot);
-      // split [lo,hi) of the concatenation A[0,IA) B[0,IB) into the A part (which 0) and the B part (which 1)
-      if (which == 0) return Seg{1, lo < IA ? lo : IA, hi < IA ? hi : IA};
-      return Seg{2, (lo > IA ? lo : IA) - IA, (hi > IA ? hi : IA) - IA};
+      // B, with two images only, has the least time to land: all of it in P0; A over P1..P3
+      if (which == 1) return Seg{0, 0, 0};
+      if (phase == 0) return Seg{2, 0, IB};
+      return Seg{1, (phase - 1) * IA / 3, phase * IA / 3};
     } else if (AK) {
       if (which == 1) return Seg{0, 0, 0};
       if (phase == 0) return Seg{1, 0, IA / 2};
@@ -360,90 +366,81 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
     }
   };
 
-  // Half a slab step: the MFMAs of fragment rows [HALF*HM, HALF*HM + HM) against every B fragment,
-  // column by column, with the LDS reads that refresh dead fragments and, when PHASE >= 0, the loads
-  // the schedule puts under this half-step.  The wave issues in order, about one instruction every four
-  // cycles, and whatever sits between two MFMAs beyond the 16 cycles the first one occupies the pipe is
-  // lost: the memory instructions are dealt out one per gap between MFMAs as far as the gaps go.
-  //   HALF 0 reads the second-half A fragments of the slab being computed (slab_rd).
-  //   HALF 1 reads, from the next slab slab_rd, the first-half A fragments and, after the last MFMA
-  //   that uses it, each B fragment.  An MN-major B fragment takes two reads: the second one goes
-  //   after the first MFMA of the next column; that of the last column is left to the HALF 0 step that
-  //   follows (PEND), which reads from the same slab.
-  // ia / ib: image (offset in the operand's region) the fragments are read from;
-  // dst_a / dst_b: LDS address of the image the A / B loads of this half-step go to.
-  auto half_step = [&](auto half, auto do_read, auto pend, int slab_rd, uint32_t ia, uint32_t ib, auto phase,
-                       uint32_t dst_a, uint32_t dst_b) {
-    constexpr int HALF = decltype(half)::value, PHASE = decltype(phase)::value;
-    constexpr bool READ = decltype(do_read)::value, PEND = decltype(pend)::value;
-    constexpr Seg s0 = PHASE >= 0 ? plan(PHASE, 0) : Seg{0, 0, 0}, s1 = PHASE >= 0 ? plan(PHASE, 1) : Seg{0, 0, 0};
-    constexpr int n0l = s0.hi - s0.lo, n1l = s1.hi - s1.lo, NL = n0l + n1l;
-    constexpr int APC = (HM + TN - 1) / TN;  // A fragments refreshed per column
-    constexpr bool SPLIT_B = !BK && HM >= 2;  // B fragment reads in two halves, one gap apart
-    i32x4 ra, rb;
-    if constexpr (NL > 0) {
-      ra = opa.rsrc();
-      rb = opb.rsrc();
-    }
-    // the l-th load of this half-step
-    auto issue = [&](auto lc) {
-      constexpr int l = decltype(lc)::value;
-      constexpr Seg sg = l < n0l ? s0 : s1;
-      constexpr int J = l < n0l ? s0.lo + l : s1.lo + (l - n0l);
-      constexpr bool first = (l == 0) || (l == n0l) || (J % 4 == 0);
-      if constexpr (sg.op == 1) {
-        if constexpr (first) dma_set_m0(dst_a + opa.lds_w + (J / 4) * 4096);
-        opa.template issue_one<J>(ra);
+  // One slab step: the TM x TN MFMAs of the slab whose fragments are in copy PAR, with the LDS reads
+  // that fetch the next slab's fragments into the other copy (READ) and the loads the schedule puts
+  // under the two halves of this step (phases PH0, PH1; -1: none).  The wave issues in order, about
+  // one instruction every four cycles, and whatever sits between two MFMAs beyond the 16 cycles the
+  // first one occupies the pipe is lost.  The four waves run in lockstep and share one LDS pipe, which
+  // takes longer than those 16 cycles over their four simultaneous 1 KiB reads: so the reads go into
+  // every other gap between MFMAs (the first three quarters of the step), the loads into gaps between.
+  //   slab_rd: the slab read from LDS (its parity picks the half of a K-major tile image);
+  //   ia / ib: image (offset in the operand's region) the fragments are read from;
+  //   dst_*0 / dst_*1: LDS address of the image the A / B loads of the first / second half go to.
+  auto slab_step = [&](auto par, auto do_read, int slab_rd, uint32_t ia, uint32_t ib, auto ph0, auto ph1,
+                       uint32_t dst_a0, uint32_t dst_b0, uint32_t dst_a1, uint32_t dst_b1) {
+    constexpr int PAR = decltype(par)::value, PH0 = decltype(ph0)::value, PH1 = decltype(ph1)::value;
+    constexpr bool READ = decltype(do_read)::value;
+    constexpr int NM = TM * TN;
+    // LDS read operations: a K-major fragment is one 16-byte read, an MN-major one two transposing
+    // 8-byte reads; A and B alternate as long as both last
+    constexpr int RA = AK ? 1 : 2, RB = BK ? 1 : 2, NRA = TM * RA, NRB = TN * RB, NR = READ ? NRA + NRB : 0;
+    constexpr int RSPAN = NM - NM / 4;
+    uint32_t base_a = 0, base_b = 0;
+    if constexpr (READ && AK) base_a = fa.base(ia, slab_rd);
+    if constexpr (READ && BK) base_b = fb.base(ib, slab_rd);
+    auto read_op = [&](auto kc) {
+      constexpr int k = decltype(kc)::value;
+      // k-th read: alternate B, A, B, A ... until one list runs out
+      constexpr int pairs = NRA < NRB ? NRA : NRB;
+      constexpr bool is_b = k < 2 * pairs ? (k % 2 == 0) : (NRB > NRA);
+      constexpr int idx = k < 2 * pairs ? k / 2 : k - pairs;
+      if constexpr (is_b) {
+        if constexpr (BK) bfr[PAR ^ 1][idx] = fb.read_at(base_b, idx);
+        else bfr[PAR ^ 1][idx / 2] = with_half(bfr[PAR ^ 1][idx / 2], fb.read_half(ib, idx / 2, idx % 2), idx % 2);
       } else {
-        if constexpr (first) dma_set_m0(dst_b + opb.lds_w + (J / 4) * 4096);
-        opb.template issue_one<J>(rb);
+        if constexpr (AK) af[PAR ^ 1][idx] = fa.read_at(base_a, idx);
+        else af[PAR ^ 1][idx / 2] = with_half(af[PAR ^ 1][idx / 2], fa.read_half(ia, idx / 2, idx % 2), idx % 2);
       }
     };
-    static_for<TN>([&](auto cc) {
-      constexpr int c = decltype(cc)::value;
-      constexpr int a_lo = c * APC < HM ? c * APC : HM, a_hi = (c + 1) * APC < HM ? (c + 1) * APC : HM;
-      constexpr int l_lo = c * NL / TN, l_hi = (c + 1) * NL / TN;  // loads spread over the TN columns
-      // memory instructions of this column in order: [second half of the previous column's B fragment]
-      // [A fragments] [loads]; the k-th goes into gap min(k, HM-1); the B read of this column always
-      // follows the column's last MFMA
-      constexpr int cprev = c == 0 ? TN - 1 : c - 1;
-      constexpr bool bhi = SPLIT_B && ((HALF == 1 && READ && c > 0) || (HALF == 0 && PEND && c == 0));
-      constexpr int nA = READ ? a_hi - a_lo : 0, nLd = l_hi - l_lo;
-      static_for<HM>([&](auto ic) {
-        constexpr int ii = decltype(ic)::value;
-        constexpr int i = HALF * HM + ii;
-        // B fragment first: D rows index n, D columns index m, so a lane ends up with 4
-        // consecutive n of one output row (an 8-byte piece) instead of 4 rows of one column.
-        mfma_16x16x32(acc[i][c], bfr[c], af[i]);
-        static_for<(bhi ? 1 : 0) + nA + nLd>([&](auto kc) {
-          constexpr int k = decltype(kc)::value;
-          if constexpr ((k < HM - 1 ? k : HM - 1) == ii) {
-            if constexpr (bhi && k == 0) {
-              bfr[cprev] = with_half(bfr[cprev], fb.read_half(ib, cprev, 1), 1);
-            } else if constexpr (k - (bhi ? 1 : 0) < nA) {
-              constexpr int f = a_lo + k - (bhi ? 1 : 0);
-              if constexpr (HALF == 0) af[HM + f] = fa.read(ia, HM + f, slab_rd);
-              else af[f] = fa.read(ia, f, slab_rd);
+    auto load_ops = [&](auto phc, auto mc, uint32_t dst_a, uint32_t dst_b, int half) {
+      constexpr int PHASE = decltype(phc)::value, m = decltype(mc)::value;  // m: gap index within the half
+      if constexpr (PHASE >= 0) {
+        constexpr Seg s0 = plan(PHASE, 0), s1 = plan(PHASE, 1);
+        constexpr int n0l = s0.hi - s0.lo, n1l = s1.hi - s1.lo, NL = n0l + n1l;
+        static_for<NL>([&](auto lc) {
+          constexpr int l = decltype(lc)::value;
+          // spread over the half, on odd gaps (the reads take the even ones)
+          constexpr int gap = (((NM / 2) * (2 * l + 1) / (2 * NL)) | 1) < NM / 2 ? (((NM / 2) * (2 * l + 1) / (2 * NL)) | 1) : NM / 2 - 1;
+          if constexpr (gap == m) {
+            constexpr Seg sg = l < n0l ? s0 : s1;
+            constexpr int J = l < n0l ? s0.lo + l : s1.lo + (l - n0l);
+            constexpr bool first = (l == 0) || (l == n0l) || (J % 4 == 0);
+            if constexpr (sg.op == 1) {
+              if constexpr (first) dma_set_m0(dst_a + opa.lds_w + (J / 4) * 4096);
+              opa.template issue_one<J>(opa.rsrc());
+              if constexpr (J == IA - 1) opa.advance();  // the unit is complete: move along K
             } else {
-              issue(std::integral_constant<int, l_lo + k - (bhi ? 1 : 0) - nA>{});
+              if constexpr (first) dma_set_m0(dst_b + opb.lds_w + (J / 4) * 4096);
+              opb.template issue_one<J>(opb.rsrc());
+              if constexpr (J == IB - 1) opb.advance();
             }
           }
         });
-      });
-      if constexpr (READ && HALF == 1) {
-        if constexpr (SPLIT_B) {
-          bfr[c] = with_half(bfr[c], fb.read_half(ib, c, 0), 0);
-          if constexpr (c == TN - 1 && !PEND) bfr[c] = with_half(bfr[c], fb.read_half(ib, c, 1), 1);
-        } else {
-          bfr[c] = fb.read(ib, c, slab_rd);
-        }
       }
+    };
+    static_for<NM>([&](auto mc) {
+      constexpr int m = decltype(mc)::value;
+      constexpr int c = m / TM, i = m % TM;
+      // B fragment first: D rows index n, D columns index m, so a lane ends up with 4
+      // consecutive n of one output row (an 8-byte piece) instead of 4 rows of one column.
+      mfma_16x16x32(acc[i][c], bfr[PAR][c], af[PAR][i]);
+      static_for<NR>([&](auto kc) {
+        constexpr int k = decltype(kc)::value;
+        if constexpr (k * RSPAN / (NR > 0 ? NR : 1) == m) read_op(kc);
+      });
+      if constexpr (m < NM / 2) load_ops(ph0, std::integral_constant<int, m>{}, dst_a0, dst_b0, 0);
+      else load_ops(ph1, std::integral_constant<int, m - NM / 2>{}, dst_a1, dst_b1, 1);
     });
-    // the unit of an operand is complete once its last load is out: move its resource along K
-    if constexpr (NL > 0) {
-      if constexpr ((s0.op == 1 && s0.hi == IA && n0l > 0) || (s1.op == 1 && s1.hi == IA && n1l > 0)) opa.advance();
-      if constexpr ((s0.op == 2 && s0.hi == IB && n0l > 0) || (s1.op == 2 && s1.hi == IB && n1l > 0)) opb.advance();
-    }
   };
 
   // All loads of one unit of an operand in a burst (prologue and tail).  `unit` counts tiles for a
@@ -499,14 +496,11 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
   };
   using T = std::true_type;
   using F = std::false_type;
-  using H0 = std::integral_constant<int, 0>;
-  using H1 = std::integral_constant<int, 1>;
-  using NoLoads = std::integral_constant<int, -1>;
 
   // One iteration j of the rotated loop is: sync, second half of slab j, first half of slab j+1.
   // After the sync every wave holds all fragments of slab j in registers and slab j+1 has landed, so
   //   an MN-major slab image j & 3 is dead and takes slab j+4;
-  //   for odd j the K-major tile image (j >> 1) % TU is dead and takes tile (j >> 1) + TU.
+  //   for odd j the K-major tile image (j >> 1) % U (U images) is dead and takes tile (j >> 1) + U.
   // Steady state, period t (iterations j = 2t+1 and 2t+2), what is issued and what each sync keeps in
   // flight (loads complete in issue order):
   //   one K-major operand X (three images), the other Y MN-major:
@@ -514,9 +508,10 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
   //     P2 = second half of slab 2t+2: Y slab 2t+5                   P3 = first half of slab 2t+3: Y slab 2t+6
   //     the sync before P0 needs X tile t+1 and Y slab 2t+2: all but the loads of the period before
   //     the sync before P2 needs Y slab 2t+3: all but Y slab 2t+4 and X tile t+3
-  //   both K-major (two images): tile t+2 of both over P0..P2; only the sync before P0 is needed, and
-  //   it needs everything
-  constexpr int KEEP_ODD = (AK && BK) ? 0 : (IA + IB + (AK ? IB : IA));
+  //   both K-major (A three images, B two): P0: B tile t+2, P1..P3: A tile t+3
+  //     the sync before P0 needs A tile t+1 and B tile t+1: all but A tile t+2
+  //     no loads land between the sync before P0 and the reads of slab 2t+3: no second sync
+  constexpr int KEEP_ODD = (AK && BK) ? IA : (IA + IB + (AK ? IB : IA));
   constexpr int KEEP_EVEN = (AK && BK) ? -1 : IA + IB;
 
   // prologue: two tiles / four slabs of each operand, all landed
@@ -526,57 +521,65 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
 #pragma unroll
-  for (int t = 0; t < HM; ++t) af[t] = fa.read(img_a(0), t, 0);
+  for (int t = 0; t < TM; ++t) af[0][t] = fa.read(img_a(0), t, 0);
 #pragma unroll
-  for (int t = 0; t < TN; ++t) bfr[t] = fb.read(img_b(0), t, 0);
-  half_step(H0{}, T{}, F{}, 0, img_a(0), img_b(0), NoLoads{}, 0, 0);
+  for (int t = 0; t < TN; ++t) bfr[0][t] = fb.read(img_b(0), t, 0);
 
+  using P0 = std::integral_constant<int, 0>;
+  using P1 = std::integral_constant<int, 1>;
+  using NoLoads = std::integral_constant<int, -1>;
   // iteration with loads in a burst and full waits: j = 0, and the tail
-  auto slow_iteration = [&](int j) {
+  auto slow_iteration = [&](auto par, int j) {
     sync(std::integral_constant<int, 0>{});
     if constexpr (!AK) { if (j + 4 < nslab) burst_a(j + 4); }
     if constexpr (!BK) { if (j + 4 < nslab) burst_b(j + 4); }
     if (j & 1) {
-      if constexpr (AK) { if ((j >> 1) + TU < ntile) burst_a((j >> 1) + TU); }
-      if constexpr (BK) { if ((j >> 1) + TU < ntile) burst_b((j >> 1) + TU); }
+      if constexpr (AK) { if ((j >> 1) + OpA::UNITS < ntile) burst_a((j >> 1) + OpA::UNITS); }
+      if constexpr (BK) { if ((j >> 1) + OpB::UNITS < ntile) burst_b((j >> 1) + OpB::UNITS); }
     }
-    half_step(H1{}, T{}, T{}, j + 1, img_a(j + 1), img_b(j + 1), NoLoads{}, 0, 0);
-    half_step(H0{}, T{}, T{}, j + 1, img_a(j + 1), img_b(j + 1), NoLoads{}, 0, 0);
+    slab_step(par, T{}, j + 1, img_a(j + 1), img_b(j + 1), NoLoads{}, NoLoads{}, 0, 0, 0, 0);
   };
-  slow_iteration(0);
+  slow_iteration(P0{}, 0);
 
   int j = 1;
   // steady: two periods per trip (the MN-major slab images repeat every four slabs, the K-major
   // tile images rotate at run time); every unit loaded here exists and is full
-  uint32_t x_ld = 0, x_rd = 1;  // tile image that takes tile t+TU (= image of tile t) / that holds tile t+1
+  uint32_t x_ld = 0, x_rd = 1;  // of three tile images: the one that takes tile t+3 (= image of tile t) / that holds tile t+1
   for (; (j >> 1) + 4 < ntile - 1; j += 4) {
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       // period t = (j >> 1) + u, t & 1 == u since j == 1 (mod 4)
       const int jo = j + 2 * u;  // the odd slab 2t+1
-      // slab images (2t+1) & 3 and (2t+2) & 3 take slabs 2t+5 and 2t+6; slabs 2t+2, 2t+3 are read
-      const uint32_t da0 = lds0 + (AK ? x_ld : (uint32_t)((2 * u + 1) & 3)) * OpA::IMG;
-      const uint32_t da1 = lds0 + (AK ? x_ld : (uint32_t)((2 * u + 2) & 3)) * OpA::IMG;
-      const uint32_t db0 = lds0 + A_BYTES + (BK ? x_ld : (uint32_t)((2 * u + 1) & 3)) * OpB::IMG;
-      const uint32_t db1 = lds0 + A_BYTES + (BK ? x_ld : (uint32_t)((2 * u + 2) & 3)) * OpB::IMG;
-      const uint32_t ra0 = (AK ? x_rd : (uint32_t)((2 * u + 2) & 3)) * OpA::IMG;
-      const uint32_t ra1 = (AK ? x_rd : (uint32_t)((2 * u + 3) & 3)) * OpA::IMG;
-      const uint32_t rb0 = (BK ? x_rd : (uint32_t)((2 * u + 2) & 3)) * OpB::IMG;
-      const uint32_t rb1 = (BK ? x_rd : (uint32_t)((2 * u + 3) & 3)) * OpB::IMG;
+      // image index for loads in the first / second half of the period and for reads of slabs 2t+2 / 2t+3:
+      //   four slab images: slabs 2t+5, 2t+6 go to (2t+1) & 3, (2t+2) & 3
+      //   three tile images: rotate at run time; two: tile t+2 goes to t & 1, tile t+1 is read
+      auto idx = [&](int units, int ld_or_rd, int second) -> uint32_t {
+        if (units == 4) return (uint32_t)((2 * u + 1 + ld_or_rd + second) & 3);
+        if (units == 3) return ld_or_rd ? x_rd : x_ld;
+        return (uint32_t)((u + ld_or_rd) & 1);
+      };
+      const uint32_t da0 = lds0 + idx(OpA::UNITS, 0, 0) * OpA::IMG, da1 = lds0 + idx(OpA::UNITS, 0, 1) * OpA::IMG;
+      const uint32_t db0 = lds0 + A_BYTES + idx(OpB::UNITS, 0, 0) * OpB::IMG,
+                     db1 = lds0 + A_BYTES + idx(OpB::UNITS, 0, 1) * OpB::IMG;
+      const uint32_t ra0 = idx(OpA::UNITS, 1, 0) * OpA::IMG, ra1 = idx(OpA::UNITS, 1, 1) * OpA::IMG;
+      const uint32_t rb0 = idx(OpB::UNITS, 1, 0) * OpB::IMG, rb1 = idx(OpB::UNITS, 1, 1) * OpB::IMG;
       sync(std::integral_constant<int, KEEP_ODD>{});
-      half_step(H1{}, T{}, T{}, jo + 1, ra0, rb0, std::integral_constant<int, 0>{}, da0, db0);
-      half_step(H0{}, T{}, T{}, jo + 1, ra0, rb0, std::integral_constant<int, 1>{}, da0, db0);
+      slab_step(P1{}, T{}, jo + 1, ra0, rb0, std::integral_constant<int, 0>{}, std::integral_constant<int, 1>{}, da0, db0,
+                da0, db0);
       if constexpr (KEEP_EVEN >= 0) sync(std::integral_constant<int, KEEP_EVEN>{});
-      half_step(H1{}, T{}, T{}, jo + 2, ra1, rb1, std::integral_constant<int, 2>{}, da0, db0);
-      half_step(H0{}, T{}, T{}, jo + 2, ra1, rb1, std::integral_constant<int, 3>{}, da1, db1);
+      slab_step(P0{}, T{}, jo + 2, ra1, rb1, std::integral_constant<int, 2>{}, std::integral_constant<int, 3>{}, da0, db0,
+                da1, db1);
       x_ld = x_rd;
-      x_rd = x_rd + 1 == TU ? 0 : x_rd + 1;
+      x_rd = x_rd + 1 == 3 ? 0 : x_rd + 1;
     }
   }
-  for (; j + 1 < nslab; ++j) slow_iteration(j);
-  // second half of the last slab: its fragments are in registers or on their way from LDS; every
-  // load was waited for by the last sync
-  half_step(H1{}, F{}, F{}, 0, 0, 0, NoLoads{}, 0, 0);
+  // j is odd and nslab even: the tail is whole pairs of iterations
+  for (; j + 1 < nslab; j += 2) {
+    slow_iteration(P1{}, j);
+    slow_iteration(P0{}, j + 1);
+  }
+  // the last slab (odd): its fragments are in registers or on their way from LDS
+  slab_step(P1{}, F{}, 0, 0, 0, NoLoads{}, NoLoads{}, 0, 0, 0, 0);
 
   // The last MFMAs must have left the pipe before their accumulators are read, and the compiler,
   // which sees neither MFMAs nor hazard here, inserts nothing.  Volatile asm statements keep their
@@ -758,8 +761,8 @@ static const VariantInfo kVariants[NEOGEMM_VARIANT_COUNT] = {
 
 template <int BM, int BN, int WGM, int WGN>
 static hipError_t launch_tile(const TileArgs& a, bool ak, bool bk, hipStream_t st) {
-  // four 32-deep images of an MN-major operand; three 64-deep ones of a K-major operand next to it, two if both are K-major
-  const size_t lds = (ak && bk) ? (size_t)(BM + BN) * 256 : (size_t)(ak ? BM : BN) * 384 + (size_t)(ak ? BN : BM) * 256;
+  // A: three 64-deep images if K-major, else four 32-deep ones; B likewise, but two 64-deep ones if both are K-major
+  const size_t lds = (size_t)BM * (ak ? 384 : 256) + (size_t)BN * (bk && !ak ? 384 : 256);
   dim3 grid(a.ntm * a.ntn, a.ksplit), block(WGM * WGN * 64);
   auto go = [&](auto kern) -> hipError_t {
     static bool attr_done = false;  // per instantiation
