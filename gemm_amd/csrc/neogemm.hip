@@ -594,6 +594,13 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
 
   // Epilogue: lane holds, per 16x16 tile, output row (lane & 15) and 4 consecutive columns 4*(lane >> 4)..+3.
   const int row_l = lane & 15, colq = (lane >> 4) * 4;
+  // An accumulator element is read out of its AGPR where it is used: left to itself the compiler copies
+  // all 256 accumulators to VGPRs ahead of the three epilogue variants below, and spills.
+  auto acc_get = [](float a) -> float {
+    float v;
+    asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(a));
+    return v;
+  };
   // Coalesced path: the wave parks its bf16 tile in LDS (the slab ring is dead by now) and reads it back
   // row-wise, so that a store instruction writes whole rows of the wave tile, 16 bytes per lane, instead of
   // sixteen 32-byte pieces.  The staging tile is WTM x WTN bf16, 16-byte chunks XOR-ed with the row number
@@ -617,7 +624,7 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
         for (int j = 0; j < TN; ++j) {
           bf16x4 o;
 #pragma unroll
-          for (int r = 0; r < 4; ++r) o[r] = (__bf16)acc[i][j][r];
+          for (int r = 0; r < 4; ++r) o[r] = (__bf16)acc_get(acc[i][j][r]);
           const uint32_t c = 2 * j + (lane >> 5);
           const uint32_t addr = region + row * (WTN * 2) + ((c ^ (row & (CH - 1))) << 4) + (((lane >> 4) & 1) << 3);
           *((NEOGEMM_AS3 bf16x4*)(uintptr_t)addr) = o;
@@ -635,7 +642,8 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
         if (grow < p.M) {
           char* dst = p.C + ((size_t)grow * p.ldc + col) * 2;
           if (col + 7 < p.N) {
-            *(bf16x8*)dst = v;
+            // C is written once and not read again here: streaming stores leave the L2 to A and B
+            __builtin_nontemporal_store(v, (bf16x8*)dst);
           } else {
 #pragma unroll
             for (int e = 0; e < 8; ++e)
@@ -655,9 +663,9 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
         const int col = n0 + wn * WTN + j * 16 + colq;
         bf16x4 o;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) o[r] = (__bf16)acc[i][j][r];
+        for (int r = 0; r < 4; ++r) o[r] = (__bf16)acc_get(acc[i][j][r]);
         if (col + 3 < p.N) {
-          *(bf16x4*)(crow + (size_t)col * 2) = o;
+          __builtin_nontemporal_store(o, (bf16x4*)(crow + (size_t)col * 2));
         } else {
 #pragma unroll
           for (int r = 0; r < 4; ++r)
@@ -676,12 +684,15 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
         const int col = n0 + wn * WTN + j * 16 + colq;
+        f32x4 o;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o[r] = acc_get(acc[i][j][r]);
         if (vec && col + 3 < p.N) {
-          *(f32x4*)(wrow + col) = acc[i][j];
+          *(f32x4*)(wrow + col) = o;
         } else {
 #pragma unroll
           for (int r = 0; r < 4; ++r)
-            if (col + r < p.N) wrow[col + r] = acc[i][j][r];
+            if (col + r < p.N) wrow[col + r] = o[r];
         }
       }
     }
