@@ -469,7 +469,6 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
     });
     opb.advance();
   };
-  const int nunit_a = AK ? ntile : nslab, nunit_b = BK ? ntile : nslab;
 
   // Wait until this wave's loads of the slab about to be read have landed (all but the `keep` most
   // recent loads), and its own LDS reads are done; then meet the other waves.
@@ -514,10 +513,19 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
   constexpr int KEEP_ODD = (AK && BK) ? IA : (IA + IB + (AK ? IB : IA));
   constexpr int KEEP_EVEN = (AK && BK) ? -1 : IA + IB;
 
-  // prologue: two tiles / four slabs of each operand, all landed
-  for (int u = 0; u < OpA::UNITS && u < nunit_a; ++u) burst_a(u);
-  for (int u = 0; u < OpB::UNITS && u < nunit_b; ++u) burst_b(u);
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  // prologue: every image of both operands is requested, what slabs 0 and 1 need first, and only that
+  // is waited for (units past K are requested too, fully masked: the counts below hold for any K).
+  //   K-major A next to MN-major B: A0 B0 B1 | A1 B2 B3 A2      (mirrored if B is the K-major one)
+  //   both K-major:                 A0 B0 | A1 B1 A2
+  constexpr int KEEP_PRO = (AK && BK) ? 2 * IA + IB : 2 * IA + 2 * IB;
+  if constexpr (AK && BK) {
+    burst_a(0); burst_b(0); burst_a(1); burst_b(1); burst_a(2);
+  } else if constexpr (AK) {
+    burst_a(0); burst_b(0); burst_b(1); burst_a(1); burst_b(2); burst_b(3); burst_a(2);
+  } else {
+    burst_b(0); burst_a(0); burst_a(1); burst_b(1); burst_a(2); burst_a(3); burst_b(2);
+  }
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(KEEP_PRO) : "memory");
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
 #pragma unroll
@@ -529,8 +537,8 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
   using P1 = std::integral_constant<int, 1>;
   using NoLoads = std::integral_constant<int, -1>;
   // iteration with loads in a burst and full waits: j = 0, and the tail
-  auto slow_iteration = [&](auto par, int j) {
-    sync(std::integral_constant<int, 0>{});
+  auto slow_iteration = [&](auto par, auto keep, int j) {
+    sync(keep);
     if constexpr (!AK) { if (j + 4 < nslab) burst_a(j + 4); }
     if constexpr (!BK) { if (j + 4 < nslab) burst_b(j + 4); }
     if (j & 1) {
@@ -539,7 +547,7 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
     }
     slab_step(par, T{}, j + 1, img_a(j + 1), img_b(j + 1), NoLoads{}, NoLoads{}, 0, 0, 0, 0);
   };
-  slow_iteration(P0{}, 0);
+  slow_iteration(P0{}, std::integral_constant<int, KEEP_PRO>{}, 0);  // nothing was issued since the prologue's wait
 
   int j = 1;
   // steady: two periods per trip (the MN-major slab images repeat every four slabs, the K-major
@@ -575,8 +583,8 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
   }
   // j is odd and nslab even: the tail is whole pairs of iterations
   for (; j + 1 < nslab; j += 2) {
-    slow_iteration(P1{}, j);
-    slow_iteration(P0{}, j + 1);
+    slow_iteration(P1{}, std::integral_constant<int, 0>{}, j);
+    slow_iteration(P0{}, std::integral_constant<int, 0>{}, j + 1);
   }
   // the last slab (odd): its fragments are in registers or on their way from LDS
   slab_step(P1{}, F{}, 0, 0, 0, NoLoads{}, NoLoads{}, 0, 0, 0, 0);
