@@ -42,13 +42,14 @@ extern "C" {
 /* Kernel variants for neogemm_bf16_variant(); 0 lets the library choose. */
 #define NEOGEMM_VARIANT_AUTO 0
 #define NEOGEMM_VARIANT_GENERIC 1   /* scalar-load fallback: any shape, stride, alignment */
-#define NEOGEMM_VARIANT_T256x256_W8 2 /* 256x256x64 macro-tile, 8 wave64 (2x4), 32x32x16 MFMA */
-#define NEOGEMM_VARIANT_T256x256_W4 3 /* 256x256x64 macro-tile, 4 wave64 (2x2) */
-#define NEOGEMM_VARIANT_T128x128_W4 4 /* 128x128x64 macro-tile, 4 wave64 (2x2) */
-#define NEOGEMM_VARIANT_T256x128_W8 5 /* 256x128x64 macro-tile, 8 wave64 (4x2) */
-#define NEOGEMM_VARIANT_T128x256_W8 6 /* 128x256x64 macro-tile, 8 wave64 (2x4) */
-#define NEOGEMM_VARIANT_T64x128_W4 7  /* 64x128x32 macro-tile, 4 wave64 (1x4), 6-slab ring: streaming, M <= 64 */
-#define NEOGEMM_VARIANT_T128x128_W4S 8 /* 128x128x32 macro-tile, 4 wave64 (1x4), 5-slab ring: streaming, M <= 128 */
+/* Tile variants: BM x BN macro-tile per workgroup, K in steps of 64, 16x16x32 MFMA; (r x c) = wave grid. */
+#define NEOGEMM_VARIANT_T256x256_W8 2 /* 256x256, 8 wave64 (2x4) */
+#define NEOGEMM_VARIANT_T256x256_W4 3 /* 256x256, 4 wave64 (2x2): the default for large shapes */
+#define NEOGEMM_VARIANT_T128x128_W4 4 /* 128x128, 4 wave64 (2x2) */
+#define NEOGEMM_VARIANT_T256x128_W8 5 /* 256x128, 8 wave64 (4x2) */
+#define NEOGEMM_VARIANT_T128x256_W8 6 /* 128x256, 8 wave64 (2x4) */
+#define NEOGEMM_VARIANT_T64x128_W4 7  /* 64x128, 4 wave64 (1x4) */
+#define NEOGEMM_VARIANT_T128x128_W4S 8 /* 128x128, 4 wave64 (1x4) */
 #define NEOGEMM_VARIANT_COUNT 9
 
 /*
