@@ -39,7 +39,7 @@ def run_abi(A, B, dev, b_layout=g.B_KN, c_layout=g.C_ROW, variant=None, split_k=
     except g.NeoGemmError as e:
         if e.status == _abi.ERR_UNSUPPORTED and variant not in (None, g.VARIANT_GENERIC) and not strict:
             # a forced tile variant may refuse a layout (an MN-major operand needs a tile >= 128 wide, ld >= tile,
-            # rows % 8 == 0; a K-major one ld >= 32): refusing is the documented behaviour, mis-running would not be
+            # rows % 8 == 0; a K-major one ld >= 64): refusing is the documented behaviour, mis-running would not be
             pytest.skip(f"variant {variant} refuses this layout/shape (status {e.status})")
         raise
     torch.cuda.synchronize()
@@ -208,6 +208,19 @@ def test_ragged_shapes_forced_tile_kernels(dev, variant, M, N, K):
             assert e.status == _abi.ERR_UNSUPPORTED and (b_layout == g.B_KN or K < 64)
             continue
         o.assert_parity(got, A, Bkn, what=f"{M}x{N}x{K} v{variant} b{b_layout}")
+
+
+# The tile kernels stage K in 64-deep tiles / 32-deep slabs with a prologue, a steady loop that is entered
+# from seven K tiles on and unrolls two periods, and a tail: every K below walks a different way through
+# them (tile counts 1..13, with and without a partial last tile), once per operand combination.
+@pytest.mark.parametrize("variant", [g.VARIANT_T256x256_W4, g.VARIANT_T256x256_W8, g.VARIANT_T128x128_W4])
+@pytest.mark.parametrize("b_layout,c_layout", [(g.B_KN, g.C_ROW), (g.B_NK, g.C_ROW), (g.B_KN, g.C_COL)])
+def test_k_loop_transitions(dev, variant, b_layout, c_layout):
+    M, N = 264, 392   # two tile rows/columns of the largest tile, ragged, both multiples of 8
+    for K in (64, 72, 120, 128, 136, 192, 200, 256, 320, 384, 440, 448, 456, 512, 576, 640, 704, 768, 776, 832):
+        A, Bkn = o.make_inputs(M, N, K, seed=K)
+        got = run_abi(A, layouts(Bkn, b_layout), dev, b_layout, c_layout, variant)
+        o.assert_parity(got, A, Bkn, what=f"{M}x{N}x{K} v{variant} b{b_layout} c{c_layout}")
 
 
 def test_k_zero_writes_zeros(dev):
