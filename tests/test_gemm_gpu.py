@@ -404,3 +404,17 @@ def test_profile_entry_point(dev):
         o.assert_parity(C, A, B, what="profiled run")
         assert lib.neogemm_bf16_profile(Ad.data_ptr(), Bd.data_ptr(), C.data_ptr(), M, N, K, K, N, N, 0, None, variant, 0,
                                         buf.data_ptr(), 8) == _abi.ERR_WORKSPACE
+
+
+def test_benchmark_driver(dev):
+    """benchmark.py (the reference driver's counterpart) on a small non-square shape: error block and timings."""
+    import io
+
+    import benchmark
+
+    out = io.StringIO()
+    st = benchmark.run(192, 320, 256, warmup=1, iters=2, seed=3, out=out)
+    assert st["rel_fro"] < 1e-3 and st["pct_within_1e-3"] > 99.0
+    text = out.getvalue()
+    assert "neoGEMM.neoGemmV1" in text and text.count("TFLOP/s") == 4
+    assert all(ms > 0 for ms in st["ms"].values())
