@@ -39,7 +39,8 @@ def _workspace(device, nbytes):
     return ws
 
 
-def gemm_into(A, B, C, M, N, K, lda, ldb, ldc, b_layout, c_layout, variant=None, split_k=0, group_m=0):
+def gemm_into(A, B, C, M, N, K, lda, ldb, ldc, b_layout, c_layout, variant=None, split_k=0, group_m=0, alpha=1.0,
+              beta=0.0):
     """Call the C ABI on torch's current stream; A, B, C are torch tensors used as device buffers."""
     need = workspace_bytes(M, N, K)
     if variant is not None and split_k > 1:
@@ -50,7 +51,7 @@ def gemm_into(A, B, C, M, N, K, lda, ldb, ldc, b_layout, c_layout, variant=None,
     with torch.cuda.device(C.device):
         stream = torch.cuda.current_stream().cuda_stream
         st = _abi.gemm_raw(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, lda, ldb, ldc, b_layout, c_layout,
-                           ws_ptr, need, stream, variant, split_k, group_m)
+                           ws_ptr, need, stream, variant, split_k, group_m, alpha, beta)
     if st != _abi.OK:
         raise NeoGemmError(st, f"M={M} N={N} K={K} b_layout={b_layout} c_layout={c_layout} variant={variant}")
 
@@ -100,3 +101,27 @@ def neoGemmV1(A, B, C, variant=None, split_k=0, group_m=0):
 
 
 neogemm = neoGemmV1
+
+
+def gemm_scaled(A, B, C, alpha=1.0, beta=0.0):
+    """C[M,N] = alpha * A[M,K] @ B[K,N] + beta * C, in place (C contiguous); neogemm_bf16_scaled."""
+    _check(A, "A")
+    _check(B, "B")
+    _check(C, "C")
+    if A.shape[1] != B.shape[0] or C.shape != (A.shape[0], B.shape[1]) or not C.is_contiguous():
+        raise ValueError(f"shapes: A {tuple(A.shape)}, B {tuple(B.shape)}, C {tuple(C.shape)} (contiguous [M,N])")
+    if A.stride(1) != 1 and A.shape[1] > 1:
+        A = A.contiguous()
+    M, K = A.shape
+    N = B.shape[1]
+    lda = A.stride(0) if M > 1 else max(K, 1)
+    if B.stride(1) == 1 or N <= 1:
+        b_layout, ldb = B_KN, (B.stride(0) if K > 1 else max(N, 1))
+    elif B.stride(0) == 1:
+        b_layout, ldb = B_NK, (B.stride(1) if N > 1 else max(K, 1))
+    else:
+        B = B.contiguous()
+        b_layout, ldb = B_KN, max(N, 1)
+    if M and N:
+        gemm_into(A, B, C, M, N, K, lda, ldb, max(N, 1), b_layout, C_ROW, alpha=float(alpha), beta=float(beta))
+    return C

@@ -24,6 +24,8 @@ VARIANT_NAMES = {0: "auto", 1: "generic", 2: "256x256_w8", 3: "256x256_w4", 4: "
 _i64, _int, _vp, _sz = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t
 PROTOTYPES = {
     "neogemm_bf16": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _vp, _sz, _vp]),
+    "neogemm_bf16_scaled": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, ctypes.c_float,
+                                   ctypes.c_float, _vp, _sz, _vp]),
     "neogemm_bf16_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "neogemm_bf16_variant": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _vp, _sz, _vp,
                                     _int, _int, _int]),
@@ -84,9 +86,14 @@ def plan(M, N, K, b_layout=B_KN, c_layout=C_ROW, aligned=True):
 
 
 def gemm_raw(A_ptr, B_ptr, C_ptr, M, N, K, lda, ldb, ldc, b_layout, c_layout, ws_ptr=0, ws_bytes=0, stream=0,
-             variant=None, split_k=0, group_m=0):
+             variant=None, split_k=0, group_m=0, alpha=1.0, beta=0.0):
     """Thin call-through; returns the status code (no exception)."""
     lib = load()
+    if alpha != 1.0 or beta != 0.0:
+        if variant is not None:
+            raise ValueError("alpha/beta go through neogemm_bf16_scaled, which chooses the kernel itself")
+        return lib.neogemm_bf16_scaled(A_ptr, B_ptr, C_ptr, M, N, K, lda, ldb, ldc, b_layout, c_layout, alpha, beta,
+                                       ws_ptr or None, ws_bytes, stream or None)
     if variant is None:
         return lib.neogemm_bf16(A_ptr, B_ptr, C_ptr, M, N, K, lda, ldb, ldc, b_layout, c_layout, ws_ptr or None,
                                 ws_bytes, stream or None)

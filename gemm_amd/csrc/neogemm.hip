@@ -115,6 +115,7 @@ struct TileArgs {
   int ntm, ntn, group_m;
   int ksplit, ktiles_per_split;  // K is cut in tiles of KTILE; a split is a run of tiles
   unsigned long long* prof;      // phase timers, 4 per wave (profiling instantiation only)
+  float alpha, beta;             // C = alpha * A*B + beta * C (beta == 0: C is not read)
 };
 
 // Global -> LDS side of one operand: which 16 bytes each lane fetches for each of this wave's
@@ -616,7 +617,7 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
   constexpr int CH = WTN / 8;        // 16-byte chunks per staged row
   constexpr int RPI = 64 / CH;       // rows one store instruction covers
   constexpr bool CAN_STAGE = (size_t)BM * BN * 2 <= (size_t)LDS_BYTES && CH >= 4 && CH <= 64;
-  const bool stage = CAN_STAGE && p.ksplit == 1 && (((uintptr_t)p.C | (uintptr_t)(p.ldc * 2)) & 15) == 0;
+  const bool stage = CAN_STAGE && p.ksplit == 1 && p.beta == 0.f && (((uintptr_t)p.C | (uintptr_t)(p.ldc * 2)) & 15) == 0;
   if (stage) {
     if constexpr (CAN_STAGE) {
       // every wave is done with the slab images (its LDS reads have returned: the MFMAs that used them
@@ -625,19 +626,27 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
       __builtin_amdgcn_s_barrier();
       asm volatile("" ::: "memory");
       const uint32_t region = lds0 + (uint32_t)wave * (WTM * WTN * 2);
+      auto park = [&](auto scaled) {
 #pragma unroll
-      for (int i = 0; i < TM; ++i) {
-        const uint32_t row = i * 16 + row_l;
+        for (int i = 0; i < TM; ++i) {
+          const uint32_t row = i * 16 + row_l;
 #pragma unroll
-        for (int j = 0; j < TN; ++j) {
-          bf16x4 o;
+          for (int j = 0; j < TN; ++j) {
+            bf16x4 o;
 #pragma unroll
-          for (int r = 0; r < 4; ++r) o[r] = (__bf16)acc_get(acc[i][j][r]);
-          const uint32_t c = 2 * j + (lane >> 5);
-          const uint32_t addr = region + row * (WTN * 2) + ((c ^ (row & (CH - 1))) << 4) + (((lane >> 4) & 1) << 3);
-          *((NEOGEMM_AS3 bf16x4*)(uintptr_t)addr) = o;
+            for (int r = 0; r < 4; ++r) {
+              float v = acc_get(acc[i][j][r]);
+              if constexpr (decltype(scaled)::value) v *= p.alpha;
+              o[r] = (__bf16)v;
+            }
+            const uint32_t c = 2 * j + (lane >> 5);
+            const uint32_t addr = region + row * (WTN * 2) + ((c ^ (row & (CH - 1))) << 4) + (((lane >> 4) & 1) << 3);
+            *((NEOGEMM_AS3 bf16x4*)(uintptr_t)addr) = o;
+          }
         }
-      }
+      };
+      if (p.alpha == 1.f) park(std::false_type{});
+      else park(std::true_type{});
       // same wave wrote and reads: LDS operations of a wave complete in order; the compiler orders them
       const int colc = lane % CH;
       const int col = n0 + wn * WTN + colc * 8;
@@ -669,9 +678,15 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
         const int col = n0 + wn * WTN + j * 16 + colq;
-        bf16x4 o;
+        f32x4 v;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) o[r] = (__bf16)acc_get(acc[i][j][r]);
+        for (int r = 0; r < 4; ++r) v[r] = acc_get(acc[i][j][r]) * p.alpha;
+        if (p.beta != 0.f) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            if (col + r < p.N) v[r] = __builtin_fmaf(p.beta, (float)*(const __bf16*)(crow + (size_t)(col + r) * 2), v[r]);
+        }
+        const bf16x4 o = {(__bf16)v[0], (__bf16)v[1], (__bf16)v[2], (__bf16)v[3]};
         if (col + 3 < p.N) {
           __builtin_nontemporal_store(o, (bf16x4*)(crow + (size_t)col * 2));
         } else {
@@ -719,8 +734,9 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
 }
 
 // Sum the split-K partials in split order (deterministic) and round once to bf16.
+// Then C = alpha * sum + beta * C.
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ ws, char* C, int M, int N,
-                                                            long ldc, int ksplit) {
+                                                            long ldc, int ksplit, float alpha, float beta) {
   const size_t MN = (size_t)M * N;
   const size_t idx = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
   if (idx >= MN) return;
@@ -734,14 +750,25 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
       s[3] += t[3];
     }
     const size_t row = idx / N, col = idx - row * N;
+    bf16x4* dst = (bf16x4*)(C + (row * ldc + col) * 2);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) s[e] *= alpha;
+    if (beta != 0.f) {
+      const bf16x4 c = *dst;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) s[e] = __builtin_fmaf(beta, (float)c[e], s[e]);
+    }
     bf16x4 o = {(__bf16)s[0], (__bf16)s[1], (__bf16)s[2], (__bf16)s[3]};
-    *(bf16x4*)(C + (row * ldc + col) * 2) = o;
+    *dst = o;
   } else {
     for (int e = 0; e < 4 && idx + e < MN; ++e) {
       float s = ws[idx + e];
       for (int z = 1; z < ksplit; ++z) s += ws[z * MN + idx + e];
       const size_t row = (idx + e) / N, col = (idx + e) - row * N;
-      *(__bf16*)(C + (row * ldc + col) * 2) = (__bf16)s;
+      __bf16* dst = (__bf16*)(C + (row * ldc + col) * 2);
+      s *= alpha;
+      if (beta != 0.f) s = __builtin_fmaf(beta, (float)*dst, s);
+      *dst = (__bf16)s;
     }
   }
 }
@@ -750,7 +777,8 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
 // One thread per output element, 16x16 outputs per workgroup, K walked 16 at a time through LDS.
 __global__ __launch_bounds__(256) void gemm_generic_kernel(const __bf16* __restrict__ A, const __bf16* __restrict__ B,
                                                            __bf16* C, int M, int N, int K, long sam, long sak,
-                                                           long sbk, long sbn, long scm, long scn) {
+                                                           long sbk, long sbn, long scm, long scn, float alpha,
+                                                           float beta) {
   __shared__ float sa[16][17];
   __shared__ float sb[16][17];
   const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
@@ -765,7 +793,12 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const __bf16* __restr
     for (int k = 0; k < 16; ++k) acc = __builtin_fmaf(sa[ty][k], sb[k][tx], acc);
     __syncthreads();
   }
-  if (row < M && col < N) C[row * scm + col * scn] = (__bf16)acc;
+  if (row < M && col < N) {
+    __bf16* dst = C + row * scm + col * scn;
+    acc *= alpha;
+    if (beta != 0.f) acc = __builtin_fmaf(beta, (float)*dst, acc);
+    *dst = (__bf16)acc;
+  }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -861,7 +894,8 @@ static void plan(int64_t M, int64_t N, int64_t K, bool aligned, int c_layout, in
 
 static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
                int64_t ldc, int b_layout, int c_layout, void* workspace, size_t workspace_bytes, void* hip_stream,
-               int variant, int split_k, int group_m, unsigned long long* prof = nullptr) {
+               int variant, int split_k, int group_m, unsigned long long* prof = nullptr, float alpha = 1.f,
+               float beta = 0.f) {
   if (M < 0 || N < 0 || K < 0) return NEOGEMM_ERR_BAD_ARG;
   if ((b_layout != NEOGEMM_B_KN && b_layout != NEOGEMM_B_NK) || (c_layout != NEOGEMM_C_ROW && c_layout != NEOGEMM_C_COL))
     return NEOGEMM_ERR_BAD_ARG;
@@ -890,7 +924,7 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
     dim3 grid(ceil_div(N, 16), ceil_div(M, 16));
     if (grid.y > 65535u * 16u) return NEOGEMM_ERR_UNSUPPORTED;
     gemm_generic_kernel<<<grid, 256, 0, st>>>((const __bf16*)A, (const __bf16*)B, (__bf16*)C, (int)M, (int)N, (int)K,
-                                              lda, 1, sbk, sbn, scm, scn);
+                                              lda, 1, sbk, sbn, scm, scn, alpha, beta);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
       fprintf(stderr, "neogemm: generic kernel launch failed: %s\n", hipGetErrorString(e));
@@ -927,10 +961,10 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
     // the planned tile is too wide for an MN-major operand: the 128x128 tile needs the least, then generic
     const int next = v != NEOGEMM_VARIANT_T128x128_W4 ? NEOGEMM_VARIANT_T128x128_W4 : NEOGEMM_VARIANT_GENERIC;
     int st = run(A, B, C, M, N, K, lda, ldb, ldc, b_layout, c_layout, workspace, workspace_bytes, hip_stream, next,
-                 next == NEOGEMM_VARIANT_GENERIC ? 1 : s, 0, nullptr);
+                 next == NEOGEMM_VARIANT_GENERIC ? 1 : s, 0, nullptr, alpha, beta);
     if (st == NEOGEMM_ERR_UNSUPPORTED && next != NEOGEMM_VARIANT_GENERIC)
       st = run(A, B, C, M, N, K, lda, ldb, ldc, b_layout, c_layout, workspace, workspace_bytes, hip_stream,
-               NEOGEMM_VARIANT_GENERIC, 1, 0, nullptr);
+               NEOGEMM_VARIANT_GENERIC, 1, 0, nullptr, alpha, beta);
     return st;
   }
   a.ntm = ceil_div(a.M, vi.bm);
@@ -943,6 +977,8 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
   a.ksplit = ceil_div(ktiles, a.ktiles_per_split);  // no empty split
   a.ws = nullptr;
   a.prof = prof;
+  a.alpha = alpha;
+  a.beta = beta;
   if (prof && (a.ksplit > 1 || vi.bm != 256 || vi.bn != 256 || !ak)) return NEOGEMM_ERR_UNSUPPORTED;
   if (a.ksplit > 1) {
     const size_t need = (size_t)a.ksplit * (size_t)M * (size_t)N * sizeof(float);
@@ -969,7 +1005,7 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
   if (a.ksplit > 1) {
     const size_t MN = (size_t)a.M * a.N;
     const unsigned blocks = (unsigned)((MN + 1023) / 1024);
-    splitk_reduce_kernel<<<blocks, 256, 0, st>>>(a.ws, a.C, a.M, a.N, a.ldc, a.ksplit);
+    splitk_reduce_kernel<<<blocks, 256, 0, st>>>(a.ws, a.C, a.M, a.N, a.ldc, a.ksplit, alpha, beta);
     e = hipGetLastError();
     if (e != hipSuccess) {
       fprintf(stderr, "neogemm: split-K reduce launch failed: %s\n", hipGetErrorString(e));
@@ -987,6 +1023,14 @@ int neogemm_bf16(const void* A, const void* B, void* C, int64_t M, int64_t N, in
                  int64_t ldc, int b_layout, int c_layout, void* workspace, size_t workspace_bytes, void* hip_stream) {
   return neogemm::run(A, B, C, M, N, K, lda, ldb, ldc, b_layout, c_layout, workspace, workspace_bytes, hip_stream,
                       NEOGEMM_VARIANT_AUTO, 0, 0);
+}
+
+int neogemm_bf16_scaled(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int64_t lda,
+                        int64_t ldb, int64_t ldc, int b_layout, int c_layout, float alpha, float beta, void* workspace,
+                        size_t workspace_bytes, void* hip_stream) {
+  if (!(alpha == alpha) || !(beta == beta)) return NEOGEMM_ERR_BAD_ARG;  // NaN scale factors
+  return neogemm::run(A, B, C, M, N, K, lda, ldb, ldc, b_layout, c_layout, workspace, workspace_bytes, hip_stream,
+                      NEOGEMM_VARIANT_AUTO, 0, 0, nullptr, alpha, beta);
 }
 
 int neogemm_bf16_variant(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int64_t lda,

@@ -48,15 +48,18 @@ torch::Tensor& workspace_for(const torch::Tensor& like, size_t bytes) {
 }
 
 void run(const torch::Tensor& A, const torch::Tensor& B, torch::Tensor& C, int64_t M, int64_t N, int64_t K,
-         int64_t lda, int64_t ldb, int64_t ldc, int b_layout, int c_layout) {
+         int64_t lda, int64_t ldb, int64_t ldc, int b_layout, int c_layout, float alpha = 1.f, float beta = 0.f) {
   // PyTorch-ROCm names its HIP devices "cuda"; these are the guard and stream accessors for that naming
   c10::hip::HIPGuardMasqueradingAsCUDA guard(A.device());
   const size_t need = neogemm_bf16_workspace_bytes(M, N, K);
   void* ws = nullptr;
   if (need) ws = workspace_for(A, need).data_ptr();
   hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(A.get_device()).stream();
-  const int st = neogemm_bf16(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, lda, ldb, ldc, b_layout, c_layout,
-                              ws, need, (void*)stream);
+  const int st = (alpha == 1.f && beta == 0.f)
+                     ? neogemm_bf16(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, lda, ldb, ldc, b_layout,
+                                    c_layout, ws, need, (void*)stream)
+                     : neogemm_bf16_scaled(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, lda, ldb, ldc, b_layout,
+                                           c_layout, alpha, beta, ws, need, (void*)stream);
   TORCH_CHECK(st == NEOGEMM_OK, "neogemm_bf16 failed: ", neogemm_strerror(st));
 }
 
@@ -86,6 +89,32 @@ torch::Tensor gemm(torch::Tensor A, torch::Tensor B) {
   return C;
 }
 
+// gemm_scaled(A, B, C, alpha, beta): C[M,N] (row-major, contiguous) = alpha * A[M,K] @ B[K,N] + beta * C, in place;
+// the epilogue the reference's v4 kernel declares (neogemmv4.cu:166,266).
+void gemm_scaled(torch::Tensor A, torch::Tensor B, torch::Tensor C, double alpha, double beta) {
+  check_operand(A, "A");
+  check_operand(B, "B");
+  check_operand(C, "C");
+  TORCH_CHECK(A.device() == B.device() && A.device() == C.device(), "A, B and C must be on the same device");
+  TORCH_CHECK(A.size(1) == B.size(0), "inner dimensions differ: A is ", A.sizes(), ", B is ", B.sizes());
+  TORCH_CHECK(C.size(0) == A.size(0) && C.size(1) == B.size(1) && C.is_contiguous(), "C must be a contiguous [M,N]");
+  if (!row_major(A)) A = A.contiguous();
+  int b_layout = NEOGEMM_B_KN;
+  int64_t ldb;
+  if (row_major(B)) {
+    ldb = row_ld(B);
+  } else if (B.stride(0) == 1) {
+    b_layout = NEOGEMM_B_NK;
+    ldb = B.size(1) <= 1 ? std::max<int64_t>(B.size(0), 1) : B.stride(1);
+  } else {
+    B = B.contiguous();
+    ldb = row_ld(B);
+  }
+  const int64_t M = A.size(0), K = A.size(1), N = B.size(1);
+  if (M == 0 || N == 0) return;
+  run(A, B, C, M, N, K, row_ld(A), ldb, std::max<int64_t>(N, 1), b_layout, NEOGEMM_C_ROW, (float)alpha, (float)beta);
+}
+
 // neoGemmV1(A, B, C): A [M,K], B [N,K], C holds M*N bf16 and receives the product column-major,
 // so that C.t() (viewing the [M,N]-shaped C of benchmark.py:12 transposed, benchmark.py:25) equals
 // A @ B.t() (benchmark.py:18) when M == N, and C.view(N, M).t() does in general.
@@ -111,5 +140,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         py::arg("C"));
   m.def("neogemm", &neoGemmV1, "alias of neoGemmV1 (the reference's first module name)", py::arg("A"),
         py::arg("B"), py::arg("C"));
+  m.def("gemm_scaled", &gemm_scaled, "C = alpha * A[M,K] @ B[K,N] + beta * C, in place", py::arg("A"), py::arg("B"),
+        py::arg("C"), py::arg("alpha") = 1.0, py::arg("beta") = 0.0);
   m.def("version", []() { return std::string(neogemm_version()); });
 }

@@ -73,6 +73,18 @@ int neogemm_bf16(const void* A, const void* B, void* C, int64_t M, int64_t N, in
                  size_t workspace_bytes, void* hip_stream);
 
 /*
+ * C = alpha * A * op(B) + beta * C: the epilogue the reference's latest kernel declares
+ * ("D = alpha*A*B + beta*C", neogemmv4.cu:166,266) and never reaches (its launch omits both
+ * factors, neogemmv4.cu:322-323).  Arguments as for neogemm_bf16.  In fp32:
+ * t = alpha * acc; if beta != 0: t = fma(beta, float(C), t); C = RNE_bf16(t).  With beta == 0 the
+ * old contents of C are not read (they may be NaN); alpha == 1, beta == 0 is neogemm_bf16 bit for bit.
+ * NaN factors are refused with NEOGEMM_ERR_BAD_ARG.
+ */
+int neogemm_bf16_scaled(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int64_t lda,
+                        int64_t ldb, int64_t ldc, int b_layout, int c_layout, float alpha, float beta,
+                        void* workspace, size_t workspace_bytes, void* hip_stream);
+
+/*
  * Upper bound of the scratch neogemm_bf16 may use for (M,N,K), in bytes.  Host-only arithmetic.
  * Counterpart of the per-call device allocations the reference's launcher makes for its TMA
  * descriptors (v01.cu:153-160, nemgemmV03.cu:60-68): here the caller owns the scratch.

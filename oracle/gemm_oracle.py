@@ -16,6 +16,7 @@ Restatements:
   ref_gemm            torch.matmul in fp32 on the CPU, rounded to bf16 — the oracle the task names.
   c_gemm / c_gemm_v1_tiles   plain C (oracle/gemm_oracle.c via ctypes): sequential-k fp32 sum, and the
                       reference's own walk (64x64x64 tiles, four k16 MMAs per slab, column-major C).
+  ref_gemm_scaled     alpha * A*B + beta * C in fp32 with one rounding (neogemm_bf16_scaled).
   exact_gemm_f64      fp64 product of the bf16 inputs: the value both fp32 orders approximate.
   f32_to_bf16_bits    round-to-nearest-even written with integer arithmetic (numpy).
 """
@@ -91,6 +92,29 @@ def ref_gemm(A, B, b_layout="kn"):
 def ref_gemm_f32(A, B, b_layout="kn"):
     Bf = B.float() if b_layout == "kn" else B.float().t()
     return torch.matmul(A.float(), Bf)
+
+
+def ref_gemm_scaled(A, B, C0, alpha, beta, b_layout="kn"):
+    """alpha * A*B + beta * C0 the way neogemm_bf16_scaled states it (the epilogue the reference's v4
+    kernel declares, neogemmv4.cu:166,266): fp32 t = alpha * acc; if beta != 0: t = fma(beta, C0, t);
+    one rounding to bf16.  With beta == 0, C0 is not looked at.  The fused multiply-add is taken in fp64
+    (beta * C0 is exact there) and rounded to fp32."""
+    acc = ref_gemm_f32(A, B, b_layout)
+    t = acc * torch.tensor(alpha, dtype=torch.float32)
+    if beta != 0.0:
+        b32 = float(torch.tensor(beta, dtype=torch.float32))
+        t = (b32 * C0.double() + t.double()).float()
+    return t.to(torch.bfloat16)
+
+
+def scaled_parity(C, A, B, C0, alpha, beta, b_layout="kn"):
+    """(max error in bf16 ulps at max(|ref|, 2^-7 rms), relative Frobenius error) of C against ref_gemm_scaled."""
+    ref = ref_gemm_scaled(A, B, C0, alpha, beta, b_layout).double()
+    Cc = C.detach().cpu().double()
+    rms = float(torch.sqrt(torch.mean(ref * ref))) if ref.numel() else 0.0
+    mag = torch.clamp(ref.abs(), min=max(rms * 2.0 ** -7, 1e-38))
+    ulp = torch.exp2(torch.floor(torch.log2(mag)) - 7)
+    return float(((Cc - ref).abs() / ulp).max()), rel_frobenius(Cc, ref)
 
 
 def exact_gemm_f64(A, B, b_layout="kn"):

@@ -418,3 +418,68 @@ def test_benchmark_driver(dev):
     text = out.getvalue()
     assert "neoGEMM.neoGemmV1" in text and text.count("TFLOP/s") == 4
     assert all(ms > 0 for ms in st["ms"].values())
+
+
+# ------------------------------------------------------------------------------------------------
+# C = alpha * A*B + beta * C (neogemm_bf16_scaled; the epilogue of neogemmv4.cu:166,266)
+# ------------------------------------------------------------------------------------------------
+def run_scaled(A, B, C0, dev, alpha, beta, b_layout=g.B_KN, c_layout=g.C_ROW):
+    M, K = A.shape
+    N = B.shape[1] if b_layout == g.B_KN else B.shape[0]
+    Cd = (C0 if c_layout == g.C_ROW else C0.t().contiguous()).to(dev)
+    g.gemm_into(A.to(dev), B.to(dev), Cd, M, N, K, max(K, 1), max(N if b_layout == g.B_KN else K, 1),
+                max(N if c_layout == g.C_ROW else M, 1), b_layout, c_layout, alpha=alpha, beta=beta)
+    torch.cuda.synchronize()
+    C = Cd.cpu()
+    return C if c_layout == g.C_ROW else C.t().contiguous()
+
+
+def test_scaled_exact_small_integers(dev):
+    gen = torch.Generator().manual_seed(21)
+    for (M, N, K) in ((24, 40, 16), (256, 512, 128), (130, 264, 72), (16, 2048, 1024)):   # generic, tile, ragged, split-K
+        A = torch.randint(-3, 4, (M, K), generator=gen).to(torch.bfloat16)
+        B = torch.randint(-3, 4, (K, N), generator=gen).to(torch.bfloat16)
+        C0 = torch.randint(-8, 9, (M, N), generator=gen).to(torch.bfloat16)
+        for alpha, beta in ((2.0, -3.0), (0.5, 0.0), (1.0, 1.0), (0.0, 2.0)):
+            want = o.ref_gemm_scaled(A, B, C0, alpha, beta)          # exact integers / halves: order-independent
+            for b_layout in (g.B_KN, g.B_NK):
+                for c_layout in (g.C_ROW, g.C_COL):
+                    got = run_scaled(A, layouts(B, b_layout), C0, dev, alpha, beta, b_layout, c_layout)
+                    assert np.array_equal(o.bits_of(got), o.bits_of(want)), (M, N, K, alpha, beta, b_layout, c_layout)
+
+
+@pytest.mark.parametrize("M,N,K", [(512, 512, 512), (2048, 2304, 1024), (300, 520, 200), (64, 14336, 4096),
+                                   (1024, 1024, 8192), (7, 9, 8)])
+def test_scaled_parity(dev, M, N, K):
+    A, Bkn = o.make_inputs(M, N, K, seed=M + K)
+    C0 = torch.randn(M, N, generator=torch.Generator().manual_seed(N)).to(torch.bfloat16)
+    for alpha, beta in ((1.5, -0.75), (-2.0, 0.0), (1.0, 1.0)):
+        for b_layout in (g.B_KN, g.B_NK):
+            got = run_scaled(A, layouts(Bkn, b_layout), C0, dev, alpha, beta, b_layout)
+            ulp, fro = o.scaled_parity(got, A, Bkn, C0, alpha, beta)
+            # tolerance of the GEMM path itself: <= 1 bf16 ulp (floored at 2^-7 rms) and <= 1e-3 relative Frobenius
+            assert ulp <= 1.0 and fro <= 1e-3, (M, N, K, alpha, beta, b_layout, ulp, fro)
+
+
+def test_scaled_special_cases(dev):
+    M, N, K = 384, 512, 256
+    A, Bkn = o.make_inputs(M, N, K, seed=77)
+    nan = torch.full((M, N), float("nan"), dtype=torch.bfloat16)
+    plain = run_abi(A, Bkn, dev)
+    # beta == 0 never reads C; alpha == 1 is the plain GEMM bit for bit; alpha == 0, beta == 1 leaves C as it is
+    assert np.array_equal(o.bits_of(run_scaled(A, Bkn, nan, dev, 1.0, 0.0)), o.bits_of(plain))
+    got = run_scaled(A, Bkn, nan, dev, 2.0, 0.0)
+    assert torch.equal(got.float(), plain.float() * 2)               # power-of-two scaling is exact
+    C0 = torch.randn(M, N, generator=torch.Generator().manual_seed(5)).to(torch.bfloat16)
+    assert np.array_equal(o.bits_of(run_scaled(A, Bkn, C0, dev, 0.0, 1.0)), o.bits_of(C0 + 0.0))
+    lib = _abi.load()
+    Ad, Bd, Cd = A.to(dev), Bkn.to(dev), C0.to(dev)
+    st = lib.neogemm_bf16_scaled(Ad.data_ptr(), Bd.data_ptr(), Cd.data_ptr(), M, N, K, K, N, N, 0, 0, float("nan"), 0.0,
+                                 None, 0, None)
+    assert st == _abi.ERR_BAD_ARG
+    import neoGEMM
+    C1 = C0.to(dev)
+    neoGEMM.gemm_scaled(Ad, Bd, C1, alpha=1.5, beta=-0.75)
+    C2 = g.gemm_scaled(Ad, Bd, C0.to(dev), 1.5, -0.75)
+    torch.cuda.synchronize()
+    assert np.array_equal(o.bits_of(C1.cpu()), o.bits_of(C2.cpu()))

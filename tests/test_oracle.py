@@ -237,3 +237,48 @@ def test_golden_fixtures(path):
 
 def test_golden_fixtures_exist():
     assert len(glob.glob(os.path.join(HERE, "golden", "*.npz"))) >= 5
+
+
+# ------------------------------------------------------------------------------------------------
+# alpha/beta restatement (neogemm_bf16_scaled): pinned by exact integer cases and by its special cases
+# ------------------------------------------------------------------------------------------------
+def test_scaled_reduces_to_plain_gemm():
+    A, B = o.make_inputs(37, 29, 53, seed=4)
+    C0 = torch.full((37, 29), float("nan"), dtype=torch.bfloat16)   # beta == 0: never looked at
+    assert np.array_equal(o.bits_of(o.ref_gemm_scaled(A, B, C0, 1.0, 0.0)), o.bits_of(o.ref_gemm(A, B)))
+
+
+def test_scaled_exact_small_integers():
+    g = torch.Generator().manual_seed(9)
+    M, N, K = 12, 10, 7
+    Ai = torch.randint(-3, 4, (M, K), generator=g)
+    Bi = torch.randint(-3, 4, (K, N), generator=g)
+    Ci = torch.randint(-8, 9, (M, N), generator=g)
+    for alpha, beta in ((2.0, -3.0), (-1.0, 1.0), (0.0, 2.0), (4.0, 0.0), (0.5, 0.5)):
+        want = [[alpha * sum(int(Ai[i, k]) * int(Bi[k, j]) for k in range(K)) + beta * int(Ci[i, j])
+                 for j in range(N)] for i in range(M)]          # Python arithmetic: exact, |values| < 256
+        got = o.ref_gemm_scaled(Ai.to(torch.bfloat16), Bi.to(torch.bfloat16), Ci.to(torch.bfloat16), alpha, beta)
+        assert got.double().tolist() == want, (alpha, beta)
+
+
+def test_scaled_power_of_two_alpha_is_exact_scaling():
+    A, B = o.make_inputs(33, 40, 64, seed=6)
+    C0 = torch.zeros(33, 40, dtype=torch.bfloat16)
+    half = o.ref_gemm_scaled(A, B, C0, 0.5, 0.0)
+    assert np.array_equal(o.bits_of(half), o.bits_of((o.ref_gemm_f32(A, B) * 0.5).to(torch.bfloat16)))
+    assert torch.equal(half.float() * 2, o.ref_gemm(A, B).float())   # no subnormals here: exact
+
+
+def test_scaled_against_fp64_formula():
+    A, B = o.make_inputs(31, 27, 96, seed=8)
+    C0 = (torch.randn(31, 27, generator=torch.Generator().manual_seed(1))).to(torch.bfloat16)
+    alpha, beta = 1.75, -0.625
+    want = alpha * o.exact_gemm_f64(A, B) + beta * C0.double()
+    got = o.ref_gemm_scaled(A, B, C0, alpha, beta).double()
+    half_ulp = torch.exp2(torch.floor(torch.log2(want.abs().clamp_min(1e-30))) - 8)
+    slack = 8 * 2.0 ** -24 * (abs(alpha) * o.abs_gemm_f64(A, B) + abs(beta) * C0.double().abs())
+    assert bool(((got - want).abs() <= half_ulp * 1.0000001 + slack).all())
+    # a dropped beta term, a swapped sign or alpha applied to C as well must all fail this check
+    for wrong in (alpha * o.exact_gemm_f64(A, B), alpha * o.exact_gemm_f64(A, B) - beta * C0.double(),
+                  alpha * (o.exact_gemm_f64(A, B) + beta * C0.double())):
+        assert not bool(((got - wrong).abs() <= half_ulp * 1.0000001 + slack).all())
