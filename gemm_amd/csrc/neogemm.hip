@@ -741,13 +741,20 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
   const size_t idx = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
   if (idx >= MN) return;
   if ((N & 3) == 0) {
+    // up to four splits are fetched at a time (the loads of one trip are independent; one at a time the
+    // kernel would spend a memory latency per split) and added in split order
     f32x4 s = *(const f32x4*)(ws + idx);
-    for (int z = 1; z < ksplit; ++z) {
-      f32x4 t = *(const f32x4*)(ws + z * MN + idx);
-      s[0] += t[0];
-      s[1] += t[1];
-      s[2] += t[2];
-      s[3] += t[3];
+    for (int z = 1; z < ksplit; z += 4) {
+      f32x4 t[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+        if (z + k < ksplit) t[k] = *(const f32x4*)(ws + (size_t)(z + k) * MN + idx);
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+        if (z + k < ksplit) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) s[e] += t[k][e];
+        }
     }
     const size_t row = idx / N, col = idx - row * N;
     bf16x4* dst = (bf16x4*)(C + (row * ldc + col) * 2);
@@ -851,8 +858,26 @@ static bool is_aligned(const void* A, const void* B, const void* C, int64_t K, i
 
 static int ceil_div(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
 
-// Shape -> (variant, split_k).  256 CUs; a 256x256 workgroup fills one CU (128 KiB of LDS).
+// Shape -> (variant, split_k) by a small cost model, in microseconds, fitted to timings on one MI355X
+// (256 CUs).  A workgroup of variant v spends `ktile_us` of its CU per 64-deep K tile and `fixed_us` on
+// prologue + epilogue; the CUs work through ceil(workgroups / 256) of them one after the other (variants
+// with small tiles put `per_cu` on a CU at once, which hides their fixed part).  Nothing runs faster than
+// the operands stream from HBM (about 5 TB/s in practice).  Splitting K costs a second launch that reads
+// the fp32 partials back (about 5 TB/s as well) plus a few microseconds, and a slower, fp32 epilogue.
 // (M, N) as the caller states them; c_layout tells which of the two the kernel will see as its rows.
+// A workgroup has about 2.5 K tiles of loads in flight, so it cannot finish a K tile faster than 1/2.5 of
+// the round trip to where the operands come from: ~0.7 us per K tile when they stream from HBM, ~0.3 us
+// when the whole problem stays in the L2s and the last-level cache.
+struct PlanCand {
+  int variant;
+  double ktile_us, fixed_us, split_fixed_us;
+  int per_cu;
+};
+static const PlanCand kPlanCands[] = {
+    {NEOGEMM_VARIANT_T256x256_W4, 1.33, 9.0, 12.0, 1}, {NEOGEMM_VARIANT_T128x256_W8, 0.78, 6.0, 5.0, 1},
+    {NEOGEMM_VARIANT_T256x128_W8, 0.78, 6.0, 5.0, 1},  {NEOGEMM_VARIANT_T128x128_W4, 0.50, 3.0, 2.0, 2},
+    {NEOGEMM_VARIANT_T64x128_W4, 0.35, 2.5, 1.0, 2},
+};
 static void plan(int64_t M, int64_t N, int64_t K, bool aligned, int c_layout, int* variant, int* split_k) {
   if (!aligned || K == 0) {
     *variant = NEOGEMM_VARIANT_GENERIC;
@@ -861,35 +886,35 @@ static void plan(int64_t M, int64_t N, int64_t K, bool aligned, int c_layout, in
   }
   const int64_t rows = c_layout == NEOGEMM_C_ROW ? M : N, cols = c_layout == NEOGEMM_C_ROW ? N : M;
   const int64_t ktiles = ceil_div(K, KTILE);
-  int v, slots;  // slots: workgroups of this variant the 256 CUs hold at once (LDS-limited)
-  if ((int64_t)ceil_div(rows, 256) * ceil_div(cols, 256) >= 64 && rows > 128 && cols > 128) {
-    // One wave per SIMD with a 128x128 wave tile reads the least LDS per flop.
-    v = NEOGEMM_VARIANT_T256x256_W4;
-    slots = 256;
-  } else if (rows <= 128 && cols >= 2048) {
-    // skinny, streaming the wide operand: 128x256 tiles keep the most bytes in flight per workgroup
-    v = NEOGEMM_VARIANT_T128x256_W8;
-    slots = 256;
-  } else if (cols <= 128 && rows >= 2048) {
-    v = NEOGEMM_VARIANT_T256x128_W8;
-    slots = 256;
-  } else {
-    v = NEOGEMM_VARIANT_T128x128_W4;
-    slots = 512;
+  const double cus = 256.0;
+  const double bytes = 2.0 * ((double)rows * K + (double)K * cols + (double)rows * cols);
+  const double stream_us = bytes / 5.0e6, lat_us = bytes > 32e6 ? 0.7 : 0.3;
+  static const int kSplits[] = {1, 2, 3, 4, 6, 8, 12, 16, 24, 32, 48, 64};
+  double best = 1e300;
+  int bv = NEOGEMM_VARIANT_T128x128_W4, bs = 1;
+  for (const PlanCand& c : kPlanCands) {
+    // the 64x128 tile has too little in flight to stream from HBM: only for problems that stay in cache
+    if (c.variant == NEOGEMM_VARIANT_T64x128_W4 && bytes > 32e6) continue;
+    const double tiles = (double)ceil_div(rows, kVariants[c.variant].bm) * (double)ceil_div(cols, kVariants[c.variant].bn);
+    for (int sp : kSplits) {
+      if (sp > 1 && ktiles / sp < 2) break;  // at least 128 deep per split
+      const double ktps = (double)ceil_div(ktiles, sp), wgs = tiles * sp;
+      const double per_cu_wgs = __builtin_ceil(wgs / cus);
+      const double rounds = __builtin_ceil(wgs / (cus * c.per_cu));
+      double t = per_cu_wgs * ktps * c.ktile_us;
+      if (t < rounds * ktps * lat_us) t = rounds * ktps * lat_us;
+      t += rounds * (c.fixed_us + (sp > 1 ? c.split_fixed_us : 0.0));
+      if (t < stream_us) t = stream_us;
+      if (sp > 1) t += 4.0 + (4.0 * sp + 2.0) * (double)rows * (double)cols / 5.0e6;
+      if (t < best) {
+        best = t;
+        bv = c.variant;
+        bs = sp;
+      }
+    }
   }
-  const int64_t tiles = (int64_t)ceil_div(rows, kVariants[v].bm) * ceil_div(cols, kVariants[v].bn);
-  int s = 1;
-  if (tiles * 4 < slots * 3) {
-    // not enough tiles to fill the chip: split K so that one round of workgroups covers the CUs,
-    // keeping >= 4 K tiles (256 deep) per split so the pipeline has something to overlap
-    int64_t want = slots / tiles;
-    int64_t maxs = ktiles / 4 > 0 ? ktiles / 4 : 1;
-    s = (int)(want < maxs ? want : maxs);
-    if (s < 1) s = 1;
-    if (s > 64) s = 64;
-  }
-  *variant = v;
-  *split_k = s;
+  *variant = bv;
+  *split_k = bs;
 }
 
 static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
