@@ -10,9 +10,12 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stdio.h>
+#include <stdlib.h>
 
 #include <type_traits>
+#include <string>
 #include <utility>
+#include <vector>
 
 #include "neogemm.h"
 
@@ -878,7 +881,7 @@ static const PlanCand kPlanCands[] = {
     {NEOGEMM_VARIANT_T256x128_W8, 0.78, 6.0, 5.0, 1},  {NEOGEMM_VARIANT_T128x128_W4, 0.50, 3.0, 2.0, 2},
     {NEOGEMM_VARIANT_T64x128_W4, 0.35, 2.5, 1.0, 2},
 };
-static void plan(int64_t M, int64_t N, int64_t K, bool aligned, int c_layout, int* variant, int* split_k) {
+static void plan_model(int64_t M, int64_t N, int64_t K, bool aligned, int c_layout, int* variant, int* split_k) {
   if (!aligned || K == 0) {
     *variant = NEOGEMM_VARIANT_GENERIC;
     *split_k = 1;
@@ -899,10 +902,18 @@ static void plan(int64_t M, int64_t N, int64_t K, bool aligned, int c_layout, in
     for (int sp : kSplits) {
       if (sp > 1 && ktiles / sp < 2) break;  // at least 128 deep per split
       const double ktps = (double)ceil_div(ktiles, sp), wgs = tiles * sp;
-      const double per_cu_wgs = __builtin_ceil(wgs / cus);
-      const double rounds = __builtin_ceil(wgs / (cus * c.per_cu));
+      // a partial round runs on an emptier chip (more power and bandwidth per CU): measured at 0.7 of a round
+      // when nearly empty, rising to 1 when full
+      auto rounds_of = [](double x) {
+        const double full = __builtin_floor(x), frac = x - full;
+        return full + (frac > 0.0 ? 0.7 + 0.3 * frac : 0.0);
+      };
+      const double per_cu_wgs = rounds_of(wgs / cus);
+      const double rounds = rounds_of(wgs / (cus * c.per_cu));
       double t = per_cu_wgs * ktps * c.ktile_us;
-      if (t < rounds * ktps * lat_us) t = rounds * ktps * lat_us;
+      // latency knows no discount, and two latency-bound workgroups on one CU were measured to take turns
+      const double lat_floor = __builtin_ceil(wgs / cus) * ktps * lat_us;
+      if (t < lat_floor) t = lat_floor;
       t += rounds * (c.fixed_us + (sp > 1 ? c.split_fixed_us : 0.0));
       if (t < stream_us) t = stream_us;
       if (sp > 1) t += 4.0 + (4.0 * sp + 2.0) * (double)rows * (double)cols / 5.0e6;
@@ -915,6 +926,63 @@ static void plan(int64_t M, int64_t N, int64_t K, bool aligned, int c_layout, in
   }
   *variant = bv;
   *split_k = bs;
+}
+
+// Tuned choices override the model: the file named by the environment variable NEOGEMM_PLAN_TABLE, read
+// once, holds a JSON array of objects {"M":..,"N":..,"K":..,"c_layout":..,"variant":..,"split_k":..}
+// (what gemm_amd/tune.py writes; c_layout defaults to 0).  The reference fixes tile and stage counts at
+// compile time (v01.cu:275-278); this is the run-time counterpart.  Entries with an unknown variant or a
+// split below 1 are ignored, and so is an unreadable file.
+struct PlanEntry {
+  int64_t M, N, K;
+  int c_layout, variant, split_k;
+};
+static const std::vector<PlanEntry>& plan_table() {
+  static const std::vector<PlanEntry> table = [] {
+    std::vector<PlanEntry> t;
+    const char* path = getenv("NEOGEMM_PLAN_TABLE");
+    FILE* f = path && *path ? fopen(path, "rb") : nullptr;
+    if (!f) return t;
+    std::string text;
+    char buf[4096];
+    size_t n;
+    while ((n = fread(buf, 1, sizeof buf, f)) > 0) text.append(buf, n);
+    fclose(f);
+    // one object at a time: the text between '{' and the next '}' (the objects are flat)
+    size_t pos = 0;
+    while ((pos = text.find('{', pos)) != std::string::npos) {
+      const size_t end = text.find('}', pos);
+      if (end == std::string::npos) break;
+      const std::string obj = text.substr(pos, end - pos);
+      auto field = [&](const char* key, long long dflt) -> long long {
+        const std::string k = std::string("\"") + key + "\"";
+        size_t at = obj.find(k);
+        if (at == std::string::npos) return dflt;
+        at = obj.find(':', at + k.size());
+        if (at == std::string::npos) return dflt;
+        return strtoll(obj.c_str() + at + 1, nullptr, 10);
+      };
+      PlanEntry e{field("M", -1), field("N", -1), field("K", -1), (int)field("c_layout", 0), (int)field("variant", -1),
+                  (int)field("split_k", 0)};
+      if (e.M > 0 && e.N > 0 && e.K > 0 && e.variant > NEOGEMM_VARIANT_AUTO && e.variant < NEOGEMM_VARIANT_COUNT &&
+          e.split_k >= 1 && e.split_k <= 64 && (e.c_layout == NEOGEMM_C_ROW || e.c_layout == NEOGEMM_C_COL))
+        t.push_back(e);
+      pos = end + 1;
+    }
+    return t;
+  }();
+  return table;
+}
+static void plan(int64_t M, int64_t N, int64_t K, bool aligned, int c_layout, int* variant, int* split_k) {
+  if (aligned && K > 0) {
+    for (const PlanEntry& e : plan_table())
+      if (e.M == M && e.N == N && e.K == K && e.c_layout == c_layout) {
+        *variant = e.variant;
+        *split_k = e.variant == NEOGEMM_VARIANT_GENERIC ? 1 : e.split_k;
+        return;
+      }
+  }
+  plan_model(M, N, K, aligned, c_layout, variant, split_k);
 }
 
 static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,

@@ -1,0 +1,91 @@
+"""Measure (variant, split-K) candidates for given shapes on the GPU and write the winners as a plan table.
+
+    python -m gemm_amd.tune --out plan_table.json 512x512x512 256x256x8192 16x14336x4096
+    NEOGEMM_PLAN_TABLE=plan_table.json python bench.py        # the library reads the table once, at first use
+
+The table is the JSON array libneogemm.so looks up before its cost model (neogemm_bf16_plan): objects
+{"M","N","K","c_layout","variant","split_k"}.  Only shapes whose best measured candidate beats the model's
+choice by more than --margin are written.  The reference has nothing of the kind: its tile and stage
+counts are template arguments (v01.cu:275-278, 304-311).
+"""
+import argparse
+import json
+import math
+import sys
+
+import torch
+
+from . import _abi, gemm_into, plan
+from ._abi import B_KN, C_ROW, ERR_UNSUPPORTED, NeoGemmError
+
+CANDIDATE_VARIANTS = (_abi.VARIANT_T256x256_W4, _abi.VARIANT_T256x256_W8, _abi.VARIANT_T128x256_W8,
+                      _abi.VARIANT_T256x128_W8, _abi.VARIANT_T128x128_W4, _abi.VARIANT_T64x128_W4)
+CANDIDATE_SPLITS = (1, 2, 3, 4, 6, 8, 12, 16, 24, 32)
+
+
+def time_us(fn, warmup=5, iters=30):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(iters):
+        fn()
+    stop.record()
+    stop.synchronize()
+    return start.elapsed_time(stop) * 1000.0 / iters
+
+
+def tune_shape(M, N, K, nbuf=1, log=sys.stderr):
+    """Returns (model choice, its time, best choice, its time) for row-major A [M,K], B [K,N], C [M,N]."""
+    gen = torch.Generator().manual_seed(0)
+    A = (torch.randn(M, K, generator=gen) / math.sqrt(K)).to(torch.bfloat16).cuda()
+    Bs = [(torch.randn(K, N, generator=gen) / math.sqrt(K)).to(torch.bfloat16).cuda() for _ in range(nbuf)]
+    C = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+    turn = [0]
+
+    def call(variant, split):
+        turn[0] += 1
+        gemm_into(A, Bs[turn[0] % nbuf], C, M, N, K, K, N, N, B_KN, C_ROW, variant, split, 0)
+
+    model = plan(M, N, K)
+    t_model = time_us(lambda: call(None, 0))
+    best, t_best = model, t_model
+    for v in CANDIDATE_VARIANTS:
+        for s in CANDIDATE_SPLITS:
+            if s > 1 and K // (64 * s) < 2:
+                break
+            try:
+                t = time_us(lambda: call(v, s))
+            except NeoGemmError as e:
+                if e.status != ERR_UNSUPPORTED:
+                    raise
+                break
+            if t < t_best:
+                best, t_best = (v, s), t
+    print(f"{M}x{N}x{K}: model {model} {t_model:.2f} us, best {best} {t_best:.2f} us", file=log)
+    return model, t_model, best, t_best
+
+
+def main():
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("shapes", nargs="+", help="MxNxK")
+    ap.add_argument("--out", required=True)
+    ap.add_argument("--margin", type=float, default=0.03, help="minimum relative gain over the model's choice")
+    ap.add_argument("--nbuf", type=int, default=1, help="rotate this many B buffers (streaming shapes)")
+    args = ap.parse_args()
+    if not torch.cuda.is_available():
+        sys.exit("tuning needs a GPU")
+    table = []
+    for sh in args.shapes:
+        M, N, K = (int(x) for x in sh.lower().split("x"))
+        model, t_model, best, t_best = tune_shape(M, N, K, args.nbuf)
+        if best != model and t_best < t_model * (1.0 - args.margin):
+            table.append({"M": M, "N": N, "K": K, "c_layout": C_ROW, "variant": best[0], "split_k": best[1]})
+    with open(args.out, "w") as f:
+        json.dump(table, f, indent=1)
+    print(f"{len(table)} entries written to {args.out}", file=sys.stderr)
+
+
+if __name__ == "__main__":
+    main()

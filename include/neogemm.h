@@ -106,6 +106,10 @@ int neogemm_bf16_variant(const void* A, const void* B, void* C, int64_t M, int64
 /*
  * What neogemm_bf16 would pick for this call: writes the variant id and split-K factor.  Host only.
  * `aligned` is nonzero when pointers and leading dimensions satisfy the MFMA path (16-byte / 8-element).
+ * The choice comes from a cost model over the tile variants; if the environment variable
+ * NEOGEMM_PLAN_TABLE names a JSON file of tuned choices (an array of objects with the integer fields
+ * "M","N","K","c_layout","variant","split_k"; gemm_amd/tune.py writes one), an entry for the exact
+ * shape wins.  The file is read once per process.
  */
 int neogemm_bf16_plan(int64_t M, int64_t N, int64_t K, int b_layout, int c_layout, int aligned,
                       int* variant, int* split_k);

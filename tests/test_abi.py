@@ -95,3 +95,32 @@ def test_profile_bytes():
     assert lib.neogemm_bf16_profile_bytes(8192, 8192, _abi.VARIANT_T256x256_W8) == 1024 * 8 * 4 * 8
     assert lib.neogemm_bf16_profile_bytes(8192, 8192, _abi.VARIANT_T256x256_W4) == 1024 * 4 * 4 * 8
     assert lib.neogemm_bf16_profile_bytes(0, 8, _abi.VARIANT_T256x256_W4) == 0
+
+
+def test_plan_table_overrides_the_model(tmp_path):
+    """NEOGEMM_PLAN_TABLE: exact-shape entries win over the cost model; malformed entries are ignored."""
+    import json
+    import subprocess
+    import sys
+
+    table = tmp_path / "plan.json"
+    table.write_text(json.dumps([
+        {"M": 512, "N": 512, "K": 512, "c_layout": 0, "variant": _abi.VARIANT_T128x128_W4, "split_k": 2},
+        {"M": 4096, "N": 4096, "K": 4096, "variant": _abi.VARIANT_T256x256_W8, "split_k": 1},   # c_layout defaults to 0
+        {"M": 8192, "N": 8192, "K": 8192, "c_layout": 0, "variant": 99, "split_k": 1},           # unknown variant
+        {"M": 1024, "N": 1024, "K": 1024, "c_layout": 0, "variant": _abi.VARIANT_T128x128_W4, "split_k": 0},  # bad split
+    ]))
+    code = ("from gemm_amd import _abi\n"
+            "print(_abi.plan(512, 512, 512), _abi.plan(4096, 4096, 4096), _abi.plan(8192, 8192, 8192), "
+            "_abi.plan(1024, 1024, 1024), _abi.plan(512, 512, 512, c_layout=1), _abi.workspace_bytes(512, 512, 512))")
+    env = dict(os.environ, NEOGEMM_PLAN_TABLE=str(table))
+    out = subprocess.run([sys.executable, "-c", code], env=env, cwd=ROOT, capture_output=True, text=True, check=True).stdout
+    model = (_abi.plan(512, 512, 512), _abi.plan(8192, 8192, 8192), _abi.plan(1024, 1024, 1024))
+    want = ((_abi.VARIANT_T128x128_W4, 2), (_abi.VARIANT_T256x256_W8, 1), model[1], model[2],
+            _abi.plan(512, 512, 512, c_layout=1), 2 * 512 * 512 * 4)
+    assert out.strip() == " ".join(str(w) for w in want)
+    # an unreadable file changes nothing
+    env = dict(os.environ, NEOGEMM_PLAN_TABLE=str(tmp_path / "missing.json"))
+    out = subprocess.run([sys.executable, "-c", "from gemm_amd import _abi\nprint(_abi.plan(512, 512, 512))"], env=env,
+                         cwd=ROOT, capture_output=True, text=True, check=True).stdout
+    assert out.strip() == str(model[0])

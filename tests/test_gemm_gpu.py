@@ -483,3 +483,14 @@ def test_scaled_special_cases(dev):
     C2 = g.gemm_scaled(Ad, Bd, C0.to(dev), 1.5, -0.75)
     torch.cuda.synchronize()
     assert np.array_equal(o.bits_of(C1.cpu()), o.bits_of(C2.cpu()))
+
+
+def test_tuner_measures_candidates(dev):
+    """gemm_amd/tune.py: every candidate it times is a valid (variant, split) and the best is no slower than the model's."""
+    import io
+
+    from gemm_amd import tune
+
+    model, t_model, best, t_best = tune.tune_shape(256, 384, 2048, log=io.StringIO())
+    assert model == g.plan(256, 384, 2048) and best[0] in tune.CANDIDATE_VARIANTS + (model[0],) and best[1] >= 1
+    assert 0 < t_best <= t_model
