@@ -125,3 +125,29 @@ def gemm_scaled(A, B, C, alpha=1.0, beta=0.0):
     if M and N:
         gemm_into(A, B, C, M, N, K, lda, ldb, max(N, 1), b_layout, C_ROW, alpha=float(alpha), beta=float(beta))
     return C
+
+
+def gemm_batched(A, B):
+    """C[b,M,N] = A[b,M,K] @ B[b,K,N] (or B [K,N], shared by the batch) in one launch; neogemm_bf16_batched."""
+    for t, name in ((A, "A"), (B, "B")):
+        if not isinstance(t, torch.Tensor) or not t.is_cuda or t.dtype != torch.bfloat16:
+            raise TypeError(f"{name} must be a bfloat16 GPU tensor")
+    if A.dim() != 3 or B.dim() not in (2, 3) or A.shape[-1] != B.shape[-2] or (B.dim() == 3 and B.shape[0] != A.shape[0]):
+        raise ValueError(f"shapes: A {tuple(A.shape)} must be [b,M,K], B {tuple(B.shape)} [b,K,N] or [K,N]")
+    A, B = A.contiguous(), B.contiguous()
+    batch, M, K = A.shape
+    N = B.shape[-1]
+    C = torch.empty((batch, M, N), dtype=torch.bfloat16, device=A.device)
+    if batch == 0 or M == 0 or N == 0:
+        return C
+    lib = _abi.load()
+    need = int(lib.neogemm_bf16_batched_workspace_bytes(M, N, K, batch))
+    ws_ptr = _workspace(C.device, need).data_ptr() if need else 0
+    with torch.cuda.device(C.device):
+        stream = torch.cuda.current_stream().cuda_stream
+        st = lib.neogemm_bf16_batched(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, max(K, 1), max(N, 1), max(N, 1),
+                                      M * K, K * N if B.dim() == 3 else 0, M * N, batch, B_KN, C_ROW, ws_ptr or None,
+                                      need, stream or None)
+    if st != _abi.OK:
+        raise NeoGemmError(st, f"batch={batch} M={M} N={N} K={K}")
+    return C

@@ -26,6 +26,9 @@ PROTOTYPES = {
     "neogemm_bf16": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _vp, _sz, _vp]),
     "neogemm_bf16_scaled": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, ctypes.c_float,
                                    ctypes.c_float, _vp, _sz, _vp]),
+    "neogemm_bf16_batched": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int,
+                                    _vp, _sz, _vp]),
+    "neogemm_bf16_batched_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64]),
     "neogemm_bf16_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "neogemm_bf16_variant": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _vp, _sz, _vp,
                                     _int, _int, _int]),

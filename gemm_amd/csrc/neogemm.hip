@@ -119,6 +119,8 @@ struct TileArgs {
   int ksplit, ktiles_per_split;  // K is cut in tiles of KTILE; a split is a run of tiles
   unsigned long long* prof;      // phase timers, 4 per wave (profiling instantiation only)
   float alpha, beta;             // C = alpha * A*B + beta * C (beta == 0: C is not read)
+  long bsa, bsb, bsc;            // batch strides in elements; blockIdx.z is the batch index
+  int batch;
 };
 
 // Global -> LDS side of one operand: which 16 bytes each lane fetches for each of this wave's
@@ -321,8 +323,12 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
 
   OpA opa;
   OpB opb;
-  opa.init(p.A, p.lda, p.M, m0, k_begin, wave, lane);
-  opb.init(p.B, p.ldb, p.N, n0, k_begin, wave, lane);
+  // problem blockIdx.z of the batch
+  const char* gA = p.A + (size_t)blockIdx.z * p.bsa * 2;
+  const char* gB = p.B + (size_t)blockIdx.z * p.bsb * 2;
+  char* gC = p.C + (size_t)blockIdx.z * p.bsc * 2;
+  opa.init(gA, p.lda, p.M, m0, k_begin, wave, lane);
+  opb.init(gB, p.ldb, p.N, n0, k_begin, wave, lane);
   FragReader<BM, AK, TM> fa;
   FragReader<BN, BK, TN> fb;
   fa.init(lds0, wm * WTM, lane);
@@ -620,7 +626,7 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
   constexpr int CH = WTN / 8;        // 16-byte chunks per staged row
   constexpr int RPI = 64 / CH;       // rows one store instruction covers
   constexpr bool CAN_STAGE = (size_t)BM * BN * 2 <= (size_t)LDS_BYTES && CH >= 4 && CH <= 64;
-  const bool stage = CAN_STAGE && p.ksplit == 1 && p.beta == 0.f && (((uintptr_t)p.C | (uintptr_t)(p.ldc * 2)) & 15) == 0;
+  const bool stage = CAN_STAGE && p.ksplit == 1 && p.beta == 0.f && (((uintptr_t)gC | (uintptr_t)(p.ldc * 2)) & 15) == 0;
   if (stage) {
     if constexpr (CAN_STAGE) {
       // every wave is done with the slab images (its LDS reads have returned: the MFMAs that used them
@@ -660,7 +666,7 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
         const bf16x8 v = *((NEOGEMM_AS3 bf16x8*)(uintptr_t)addr);
         const int grow = m0 + wm * WTM + (int)row;
         if (grow < p.M) {
-          char* dst = p.C + ((size_t)grow * p.ldc + col) * 2;
+          char* dst = gC + ((size_t)grow * p.ldc + col) * 2;
           if (col + 7 < p.N) {
             // C is written once and not read again here: streaming stores leave the L2 to A and B
             __builtin_nontemporal_store(v, (bf16x8*)dst);
@@ -677,7 +683,7 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
     for (int i = 0; i < TM; ++i) {
       const int row = m0 + wm * WTM + i * 16 + row_l;
       if (row >= p.M) continue;
-      char* crow = p.C + (size_t)row * p.ldc * 2;
+      char* crow = gC + (size_t)row * p.ldc * 2;
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
         const int col = n0 + wn * WTN + j * 16 + colq;
@@ -700,7 +706,7 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
       }
     }
   } else {
-    float* wsz = p.ws + (size_t)kz * p.M * p.N;
+    float* wsz = p.ws + ((size_t)blockIdx.z * p.ksplit + kz) * p.M * p.N;
     const bool vec = (p.N & 3) == 0;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
@@ -739,8 +745,11 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
 // Sum the split-K partials in split order (deterministic) and round once to bf16.
 // Then C = alpha * sum + beta * C.
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ ws, char* C, int M, int N,
-                                                            long ldc, int ksplit, float alpha, float beta) {
+                                                            long ldc, int ksplit, float alpha, float beta,
+                                                            long bsc) {
   const size_t MN = (size_t)M * N;
+  ws += (size_t)blockIdx.y * ksplit * MN;  // problem blockIdx.y of the batch
+  C += (size_t)blockIdx.y * bsc * 2;
   const size_t idx = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
   if (idx >= MN) return;
   if ((N & 3) == 0) {
@@ -788,7 +797,10 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
 __global__ __launch_bounds__(256) void gemm_generic_kernel(const __bf16* __restrict__ A, const __bf16* __restrict__ B,
                                                            __bf16* C, int M, int N, int K, long sam, long sak,
                                                            long sbk, long sbn, long scm, long scn, float alpha,
-                                                           float beta) {
+                                                           float beta, long bsa, long bsb, long bsc) {
+  A += (size_t)blockIdx.z * bsa;  // problem blockIdx.z of the batch
+  B += (size_t)blockIdx.z * bsb;
+  C += (size_t)blockIdx.z * bsc;
   __shared__ float sa[16][17];
   __shared__ float sb[16][17];
   const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
@@ -825,7 +837,7 @@ template <int BM, int BN, int WGM, int WGN>
 static hipError_t launch_tile(const TileArgs& a, bool ak, bool bk, hipStream_t st) {
   // A: three 64-deep images if K-major, else four 32-deep ones; B likewise, but two 64-deep ones if both are K-major
   const size_t lds = (size_t)BM * (ak ? 384 : 256) + (size_t)BN * (bk && !ak ? 384 : 256);
-  dim3 grid(a.ntm * a.ntn, a.ksplit), block(WGM * WGN * 64);
+  dim3 grid(a.ntm * a.ntn, a.ksplit, a.batch), block(WGM * WGN * 64);
   auto go = [&](auto kern) -> hipError_t {
     static bool attr_done = false;  // per instantiation
     if (!attr_done) {
@@ -881,7 +893,8 @@ static const PlanCand kPlanCands[] = {
     {NEOGEMM_VARIANT_T256x128_W8, 0.78, 6.0, 5.0, 1},  {NEOGEMM_VARIANT_T128x128_W4, 0.50, 3.0, 2.0, 2},
     {NEOGEMM_VARIANT_T64x128_W4, 0.35, 2.5, 1.0, 2},
 };
-static void plan_model(int64_t M, int64_t N, int64_t K, bool aligned, int c_layout, int* variant, int* split_k) {
+static void plan_model(int64_t M, int64_t N, int64_t K, bool aligned, int c_layout, int* variant, int* split_k,
+                       int64_t batch = 1) {
   if (!aligned || K == 0) {
     *variant = NEOGEMM_VARIANT_GENERIC;
     *split_k = 1;
@@ -890,7 +903,7 @@ static void plan_model(int64_t M, int64_t N, int64_t K, bool aligned, int c_layo
   const int64_t rows = c_layout == NEOGEMM_C_ROW ? M : N, cols = c_layout == NEOGEMM_C_ROW ? N : M;
   const int64_t ktiles = ceil_div(K, KTILE);
   const double cus = 256.0;
-  const double bytes = 2.0 * ((double)rows * K + (double)K * cols + (double)rows * cols);
+  const double bytes = 2.0 * ((double)rows * K + (double)K * cols + (double)rows * cols) * (double)batch;
   const double stream_us = bytes / 5.0e6, lat_us = bytes > 32e6 ? 0.7 : 0.3;
   static const int kSplits[] = {1, 2, 3, 4, 6, 8, 12, 16, 24, 32, 48, 64};
   double best = 1e300;
@@ -901,7 +914,7 @@ static void plan_model(int64_t M, int64_t N, int64_t K, bool aligned, int c_layo
     const double tiles = (double)ceil_div(rows, kVariants[c.variant].bm) * (double)ceil_div(cols, kVariants[c.variant].bn);
     for (int sp : kSplits) {
       if (sp > 1 && ktiles / sp < 2) break;  // at least 128 deep per split
-      const double ktps = (double)ceil_div(ktiles, sp), wgs = tiles * sp;
+      const double ktps = (double)ceil_div(ktiles, sp), wgs = tiles * sp * (double)batch;
       // a partial round runs on an emptier chip (more power and bandwidth per CU): measured at 0.7 of a round
       // when nearly empty, rising to 1 when full
       auto rounds_of = [](double x) {
@@ -916,7 +929,7 @@ static void plan_model(int64_t M, int64_t N, int64_t K, bool aligned, int c_layo
       if (t < lat_floor) t = lat_floor;
       t += rounds * (c.fixed_us + (sp > 1 ? c.split_fixed_us : 0.0));
       if (t < stream_us) t = stream_us;
-      if (sp > 1) t += 4.0 + (4.0 * sp + 2.0) * (double)rows * (double)cols / 5.0e6;
+      if (sp > 1) t += 4.0 + (4.0 * sp + 2.0) * (double)rows * (double)cols * (double)batch / 5.0e6;
       if (t < best) {
         best = t;
         bv = c.variant;
@@ -973,8 +986,9 @@ static const std::vector<PlanEntry>& plan_table() {
   }();
   return table;
 }
-static void plan(int64_t M, int64_t N, int64_t K, bool aligned, int c_layout, int* variant, int* split_k) {
-  if (aligned && K > 0) {
+static void plan(int64_t M, int64_t N, int64_t K, bool aligned, int c_layout, int* variant, int* split_k,
+                 int64_t batch = 1) {
+  if (aligned && K > 0 && batch == 1) {
     for (const PlanEntry& e : plan_table())
       if (e.M == M && e.N == N && e.K == K && e.c_layout == c_layout) {
         *variant = e.variant;
@@ -982,14 +996,25 @@ static void plan(int64_t M, int64_t N, int64_t K, bool aligned, int c_layout, in
         return;
       }
   }
-  plan_model(M, N, K, aligned, c_layout, variant, split_k);
+  plan_model(M, N, K, aligned, c_layout, variant, split_k, batch);
 }
+
+// A batch of `count` problems of one shape; strides in elements between consecutive problems (0: shared operand).
+struct BatchArgs {
+  int64_t count = 1, sa = 0, sb = 0, sc = 0;
+};
 
 static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
                int64_t ldc, int b_layout, int c_layout, void* workspace, size_t workspace_bytes, void* hip_stream,
                int variant, int split_k, int group_m, unsigned long long* prof = nullptr, float alpha = 1.f,
-               float beta = 0.f) {
+               float beta = 0.f, const BatchArgs& bt = BatchArgs()) {
   if (M < 0 || N < 0 || K < 0) return NEOGEMM_ERR_BAD_ARG;
+  if (bt.count < 1 || bt.count > 65535 || bt.sa < 0 || bt.sb < 0 || bt.sc < 0) return NEOGEMM_ERR_BAD_ARG;
+  if (bt.count > 1 && M > 0 && N > 0) {
+    // the outputs of the batch must not overlap
+    const int64_t c_extent = c_layout == NEOGEMM_C_ROW ? (M - 1) * ldc + N : (N - 1) * ldc + M;
+    if (bt.sc < c_extent) return NEOGEMM_ERR_BAD_ARG;
+  }
   if ((b_layout != NEOGEMM_B_KN && b_layout != NEOGEMM_B_NK) || (c_layout != NEOGEMM_C_ROW && c_layout != NEOGEMM_C_COL))
     return NEOGEMM_ERR_BAD_ARG;
   if (variant < 0 || variant >= NEOGEMM_VARIANT_COUNT || split_k < 0 || group_m < 0) return NEOGEMM_ERR_BAD_ARG;
@@ -1001,11 +1026,12 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
   hipStream_t st = (hipStream_t)hip_stream;
 
   // ld limits keep every in-tile byte offset below 2^31 (the buffer range check uses 32-bit offsets)
-  const bool aligned = is_aligned(A, B, C, K, lda, ldb, ldc) && lda < (1 << 21) && ldb < (1 << 21) && K > 0;
+  const bool aligned = is_aligned(A, B, C, K, lda, ldb, ldc) && lda < (1 << 21) && ldb < (1 << 21) && K > 0 &&
+                       (bt.sa & 7) == 0 && (bt.sb & 7) == 0 && (bt.sc & 3) == 0;
   int v = variant, s = split_k;
   if (v == NEOGEMM_VARIANT_AUTO) {
     int pv, ps;
-    plan(M, N, K, aligned, c_layout, &pv, &ps);
+    plan(M, N, K, aligned, c_layout, &pv, &ps, bt.count);
     v = pv;
     if (s == 0) s = ps;
   }
@@ -1014,10 +1040,10 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
   if (v == NEOGEMM_VARIANT_GENERIC) {
     const long sbk = b_layout == NEOGEMM_B_KN ? ldb : 1, sbn = b_layout == NEOGEMM_B_KN ? 1 : ldb;
     const long scm = c_layout == NEOGEMM_C_ROW ? ldc : 1, scn = c_layout == NEOGEMM_C_ROW ? 1 : ldc;
-    dim3 grid(ceil_div(N, 16), ceil_div(M, 16));
-    if (grid.y > 65535u * 16u) return NEOGEMM_ERR_UNSUPPORTED;
+    dim3 grid(ceil_div(N, 16), ceil_div(M, 16), (unsigned)bt.count);
+    if (grid.y > 65535u) return NEOGEMM_ERR_UNSUPPORTED;
     gemm_generic_kernel<<<grid, 256, 0, st>>>((const __bf16*)A, (const __bf16*)B, (__bf16*)C, (int)M, (int)N, (int)K,
-                                              lda, 1, sbk, sbn, scm, scn, alpha, beta);
+                                              lda, 1, sbk, sbn, scm, scn, alpha, beta, bt.sa, bt.sb, bt.sc);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
       fprintf(stderr, "neogemm: generic kernel launch failed: %s\n", hipGetErrorString(e));
@@ -1033,14 +1059,16 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
   TileArgs a;
   bool ak, bk;
   if (c_layout == NEOGEMM_C_ROW) {
-    a.A = (const char*)A; a.lda = lda; ak = true; a.M = (int)M;
-    a.B = (const char*)B; a.ldb = ldb; bk = (b_layout == NEOGEMM_B_NK); a.N = (int)N;
+    a.A = (const char*)A; a.lda = lda; ak = true; a.M = (int)M; a.bsa = bt.sa;
+    a.B = (const char*)B; a.ldb = ldb; bk = (b_layout == NEOGEMM_B_NK); a.N = (int)N; a.bsb = bt.sb;
   } else {
-    a.A = (const char*)B; a.lda = ldb; ak = (b_layout == NEOGEMM_B_NK); a.M = (int)N;
-    a.B = (const char*)A; a.ldb = lda; bk = true; a.N = (int)M;
+    a.A = (const char*)B; a.lda = ldb; ak = (b_layout == NEOGEMM_B_NK); a.M = (int)N; a.bsa = bt.sb;
+    a.B = (const char*)A; a.ldb = lda; bk = true; a.N = (int)M; a.bsb = bt.sa;
   }
   a.C = (char*)C;
   a.ldc = ldc;
+  a.bsc = bt.sc;
+  a.batch = (int)bt.count;
   a.K = (int)K;
   const VariantInfo& vi = kVariants[v];
   // What the tile kernels assume about an operand (see Operand::init): an MN-major tile needs >= 128
@@ -1054,10 +1082,10 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
     // the planned tile is too wide for an MN-major operand: the 128x128 tile needs the least, then generic
     const int next = v != NEOGEMM_VARIANT_T128x128_W4 ? NEOGEMM_VARIANT_T128x128_W4 : NEOGEMM_VARIANT_GENERIC;
     int st = run(A, B, C, M, N, K, lda, ldb, ldc, b_layout, c_layout, workspace, workspace_bytes, hip_stream, next,
-                 next == NEOGEMM_VARIANT_GENERIC ? 1 : s, 0, nullptr, alpha, beta);
+                 next == NEOGEMM_VARIANT_GENERIC ? 1 : s, 0, nullptr, alpha, beta, bt);
     if (st == NEOGEMM_ERR_UNSUPPORTED && next != NEOGEMM_VARIANT_GENERIC)
       st = run(A, B, C, M, N, K, lda, ldb, ldc, b_layout, c_layout, workspace, workspace_bytes, hip_stream,
-               NEOGEMM_VARIANT_GENERIC, 1, 0, nullptr, alpha, beta);
+               NEOGEMM_VARIANT_GENERIC, 1, 0, nullptr, alpha, beta, bt);
     return st;
   }
   a.ntm = ceil_div(a.M, vi.bm);
@@ -1072,9 +1100,9 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
   a.prof = prof;
   a.alpha = alpha;
   a.beta = beta;
-  if (prof && (a.ksplit > 1 || vi.bm != 256 || vi.bn != 256 || !ak)) return NEOGEMM_ERR_UNSUPPORTED;
+  if (prof && (bt.count > 1 || a.ksplit > 1 || vi.bm != 256 || vi.bn != 256 || !ak)) return NEOGEMM_ERR_UNSUPPORTED;
   if (a.ksplit > 1) {
-    const size_t need = (size_t)a.ksplit * (size_t)M * (size_t)N * sizeof(float);
+    const size_t need = (size_t)a.ksplit * (size_t)M * (size_t)N * sizeof(float) * (size_t)bt.count;
     if (!workspace || workspace_bytes < need) return NEOGEMM_ERR_WORKSPACE;
     if (((uintptr_t)workspace & 15) != 0) return NEOGEMM_ERR_BAD_ARG;
     a.ws = (float*)workspace;
@@ -1098,7 +1126,8 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
   if (a.ksplit > 1) {
     const size_t MN = (size_t)a.M * a.N;
     const unsigned blocks = (unsigned)((MN + 1023) / 1024);
-    splitk_reduce_kernel<<<blocks, 256, 0, st>>>(a.ws, a.C, a.M, a.N, a.ldc, a.ksplit, alpha, beta);
+    splitk_reduce_kernel<<<dim3(blocks, (unsigned)bt.count), 256, 0, st>>>(a.ws, a.C, a.M, a.N, a.ldc, a.ksplit, alpha, beta,
+                                                                           a.bsc);
     e = hipGetLastError();
     if (e != hipSuccess) {
       fprintf(stderr, "neogemm: split-K reduce launch failed: %s\n", hipGetErrorString(e));
@@ -1124,6 +1153,28 @@ int neogemm_bf16_scaled(const void* A, const void* B, void* C, int64_t M, int64_
   if (!(alpha == alpha) || !(beta == beta)) return NEOGEMM_ERR_BAD_ARG;  // NaN scale factors
   return neogemm::run(A, B, C, M, N, K, lda, ldb, ldc, b_layout, c_layout, workspace, workspace_bytes, hip_stream,
                       NEOGEMM_VARIANT_AUTO, 0, 0, nullptr, alpha, beta);
+}
+
+int neogemm_bf16_batched(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int64_t lda,
+                         int64_t ldb, int64_t ldc, int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t batch,
+                         int b_layout, int c_layout, void* workspace, size_t workspace_bytes, void* hip_stream) {
+  if (batch == 0) return (M < 0 || N < 0 || K < 0) ? NEOGEMM_ERR_BAD_ARG : NEOGEMM_OK;
+  neogemm::BatchArgs bt;
+  bt.count = batch;
+  bt.sa = stride_a;
+  bt.sb = stride_b;
+  bt.sc = stride_c;
+  return neogemm::run(A, B, C, M, N, K, lda, ldb, ldc, b_layout, c_layout, workspace, workspace_bytes, hip_stream,
+                      NEOGEMM_VARIANT_AUTO, 0, 0, nullptr, 1.f, 0.f, bt);
+}
+
+size_t neogemm_bf16_batched_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t batch) {
+  if (M <= 0 || N <= 0 || K <= 0 || batch <= 0) return 0;
+  int v, s, v2, s2;
+  neogemm::plan(M, N, K, true, NEOGEMM_C_ROW, &v, &s, batch);
+  neogemm::plan(M, N, K, true, NEOGEMM_C_COL, &v2, &s2, batch);
+  if (s2 > s) s = s2;
+  return s > 1 ? (size_t)s * (size_t)M * (size_t)N * sizeof(float) * (size_t)batch : 0;
 }
 
 int neogemm_bf16_variant(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int64_t lda,

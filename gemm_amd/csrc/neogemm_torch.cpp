@@ -115,6 +115,31 @@ void gemm_scaled(torch::Tensor A, torch::Tensor B, torch::Tensor C, double alpha
   run(A, B, C, M, N, K, row_ld(A), ldb, std::max<int64_t>(N, 1), b_layout, NEOGEMM_C_ROW, (float)alpha, (float)beta);
 }
 
+// bmm(A, B): A [b,M,K], B [b,K,N] or [K,N] (shared) -> new C [b,M,N]; one launch (neogemm_bf16_batched).
+torch::Tensor bmm(torch::Tensor A, torch::Tensor B) {
+  TORCH_CHECK(A.is_cuda() && B.is_cuda(), "A and B must be GPU tensors (there is no CPU path)");
+  TORCH_CHECK(A.scalar_type() == torch::kBFloat16 && B.scalar_type() == torch::kBFloat16, "A and B must be bfloat16");
+  TORCH_CHECK(A.dim() == 3 && (B.dim() == 3 || B.dim() == 2), "A must be [b,M,K], B [b,K,N] or [K,N]");
+  TORCH_CHECK(A.device() == B.device(), "A and B must be on the same device");
+  TORCH_CHECK(A.size(2) == B.size(B.dim() - 2) && (B.dim() == 2 || B.size(0) == A.size(0)), "shapes do not match: A ",
+              A.sizes(), ", B ", B.sizes());
+  A = A.contiguous();
+  B = B.contiguous();
+  const int64_t batch = A.size(0), M = A.size(1), K = A.size(2), N = B.size(B.dim() - 1);
+  torch::Tensor C = torch::empty({batch, M, N}, A.options());
+  if (batch == 0 || M == 0 || N == 0) return C;
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(A.device());
+  const size_t need = neogemm_bf16_batched_workspace_bytes(M, N, K, batch);
+  void* ws = nullptr;
+  if (need) ws = workspace_for(A, need).data_ptr();
+  hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(A.get_device()).stream();
+  const int st = neogemm_bf16_batched(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, std::max<int64_t>(K, 1),
+                                      std::max<int64_t>(N, 1), std::max<int64_t>(N, 1), M * K, B.dim() == 3 ? K * N : 0,
+                                      M * N, batch, NEOGEMM_B_KN, NEOGEMM_C_ROW, ws, need, (void*)stream);
+  TORCH_CHECK(st == NEOGEMM_OK, "neogemm_bf16_batched failed: ", neogemm_strerror(st));
+  return C;
+}
+
 // neoGemmV1(A, B, C): A [M,K], B [N,K], C holds M*N bf16 and receives the product column-major,
 // so that C.t() (viewing the [M,N]-shaped C of benchmark.py:12 transposed, benchmark.py:25) equals
 // A @ B.t() (benchmark.py:18) when M == N, and C.view(N, M).t() does in general.
@@ -142,5 +167,6 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         py::arg("B"), py::arg("C"));
   m.def("gemm_scaled", &gemm_scaled, "C = alpha * A[M,K] @ B[K,N] + beta * C, in place", py::arg("A"), py::arg("B"),
         py::arg("C"), py::arg("alpha") = 1.0, py::arg("beta") = 0.0);
+  m.def("bmm", &bmm, "C[b,M,N] = A[b,M,K] @ B[b,K,N] (or B [K,N] shared)", py::arg("A"), py::arg("B"));
   m.def("version", []() { return std::string(neogemm_version()); });
 }

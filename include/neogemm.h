@@ -85,6 +85,20 @@ int neogemm_bf16_scaled(const void* A, const void* B, void* C, int64_t M, int64_
                         void* workspace, size_t workspace_bytes, void* hip_stream);
 
 /*
+ * `batch` problems of one shape in one launch: problem b uses A + b*stride_a, B + b*stride_b,
+ * C + b*stride_c (strides in elements; 0 for A or B shares that operand across the batch; the outputs
+ * must not overlap).  Everything else as for neogemm_bf16.  The reference has no batched call — its
+ * launcher takes one (A,B,C) triple (nemgemmV03.cu:343-351); this is the same launcher over a third grid
+ * dimension.  1 <= batch <= 65535 (0 is a no-op); the workspace bound is
+ * neogemm_bf16_batched_workspace_bytes(M,N,K,batch).
+ */
+int neogemm_bf16_batched(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int64_t lda,
+                         int64_t ldb, int64_t ldc, int64_t stride_a, int64_t stride_b, int64_t stride_c,
+                         int64_t batch, int b_layout, int c_layout, void* workspace, size_t workspace_bytes,
+                         void* hip_stream);
+size_t neogemm_bf16_batched_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t batch);
+
+/*
  * Upper bound of the scratch neogemm_bf16 may use for (M,N,K), in bytes.  Host-only arithmetic.
  * Counterpart of the per-call device allocations the reference's launcher makes for its TMA
  * descriptors (v01.cu:153-160, nemgemmV03.cu:60-68): here the caller owns the scratch.

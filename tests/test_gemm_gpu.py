@@ -494,3 +494,42 @@ def test_tuner_measures_candidates(dev):
     model, t_model, best, t_best = tune.tune_shape(256, 384, 2048, log=io.StringIO())
     assert model == g.plan(256, 384, 2048) and best[0] in tune.CANDIDATE_VARIANTS + (model[0],) and best[1] >= 1
     assert 0 < t_best <= t_model
+
+
+# ------------------------------------------------------------------------------------------------
+# batched (neogemm_bf16_batched): every problem of the batch against the oracle
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("batch,M,N,K", [(3, 256, 384, 512), (5, 130, 72, 200), (2, 1024, 1024, 1024), (4, 16, 2048, 4096),
+                                         (7, 5, 9, 12), (1, 512, 512, 512)])
+def test_batched_parity(dev, batch, M, N, K):
+    As, Bs = zip(*(o.make_inputs(M, N, K, seed=100 * b + M) for b in range(batch)))
+    A, B = torch.stack(As), torch.stack(Bs)
+    C = g.gemm_batched(A.to(dev), B.to(dev))
+    torch.cuda.synchronize()
+    assert C.shape == (batch, M, N)
+    for b in range(batch):
+        o.assert_parity(C[b], As[b], Bs[b], what=f"batch {b} of {batch}x{M}x{N}x{K}")
+    # a shared B (stride 0) and the extension's entry point
+    C2 = g.gemm_batched(A.to(dev), Bs[0].to(dev))
+    import neoGEMM
+    C3 = neoGEMM.bmm(A.to(dev), B.to(dev))
+    torch.cuda.synchronize()
+    for b in range(batch):
+        o.assert_parity(C2[b], As[b], Bs[0], what=f"shared B, batch {b}")
+    assert np.array_equal(o.bits_of(C3.cpu().view(batch * M, N)), o.bits_of(C.cpu().view(batch * M, N)))
+    # one problem of the batch is the plain call bit for bit when both take the same (variant, split)
+    if g.plan(M, N, K) == tuple(_abi.plan(M, N, K)) and batch == 1:
+        assert np.array_equal(o.bits_of(C[0].cpu()), o.bits_of(g.gemm(A[0].to(dev), B[0].to(dev)).cpu()))
+
+
+def test_batched_argument_checks(dev):
+    lib = _abi.load()
+    A = torch.zeros(2, 64, 64, dtype=torch.bfloat16, device=dev)
+    C = torch.zeros(2, 64, 64, dtype=torch.bfloat16, device=dev)
+    call = lambda sc, batch: lib.neogemm_bf16_batched(A.data_ptr(), A.data_ptr(), C.data_ptr(), 64, 64, 64, 64, 64, 64,
+                                                      4096, 4096, sc, batch, 0, 0, None, 0, None)
+    assert call(4096, 2) == _abi.OK
+    assert call(100, 2) == _abi.ERR_BAD_ARG          # outputs would overlap
+    assert call(4096, 70000) == _abi.ERR_BAD_ARG     # more than 65535 problems
+    assert call(4096, 0) == _abi.OK                  # empty batch: nothing to do
+    torch.cuda.synchronize()
