@@ -742,6 +742,200 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Skinny M (decode shapes: M <= 16 * TMF, row-major C): bound by streaming B from HBM once, so what
+// counts is bytes in flight per CU, not MFMA rate.  A workgroup owns a strip of 64 columns of C and the
+// whole of K; no split-K, no second launch.  Its four waves split K between them in steps of 64 (wave w
+// takes steps w, w+4, ...), each with a private ring of RS steps in LDS that only it fills and reads:
+// no barrier until the end, when the four partial sums meet in LDS and are added in wave order.
+// One step of one wave: A 16*TMF rows x 128 B (K-major image, swz_k), B 64 k-rows x 128 B if B is [K,N]
+// (64 columns are one cache line per k-row; swizzle swz_mn64) or 64 rows x 128 B if B is [N,K].
+// 4 waves x RS steps x (2 KiB * TMF + 8 KiB) of LDS: TMF = 1, RS = 4 fills the 160 KiB; TMF = 2, RS = 3 and
+// TMF = 4, RS = 2 (M <= 64: 30.5 us at 64x14336x4096, the split-K tile path 32.9) are the other instances.
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ uint32_t swz_mn64(uint32_t kk) {
+  // k-row kk (0..31 within a slab) of a 64-column MN-major image: even values 0..6 XOR-ed into the 16-byte chunk
+  // index, chosen so that the sixteen 32-byte pieces of one transposing read spread over the banks
+  return ((((kk >> 3) & 3u) ^ (((kk >> 1) & 1u) << 1)) << 1);
+}
+struct SkinnyArgs {
+  const char* A;
+  const char* B;
+  char* C;
+  int M, N, K;
+  long lda, ldb, ldc;
+  float alpha, beta;
+};
+template <int TMF, int RS, bool BKM>
+__global__ __launch_bounds__(256) void gemm_skinny_kernel(SkinnyArgs p) {
+  constexpr int BM = 16 * TMF;
+  constexpr uint32_t A_STEP = BM * 128, B_STEP = 64 * 128, STEP = A_STEP + B_STEP;
+  constexpr int NA = A_STEP / 1024, NB = B_STEP / 1024, LP = NA + NB;  // 1 KiB loads per step
+  static_assert(4u * RS * STEP <= 160u * 1024u, "the four rings must fit the LDS");
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(NEOGEMM_AS3 char*)smem;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n0 = blockIdx.x * 64;
+  const int nsteps = (p.K + KTILE - 1) / KTILE;
+  const uint32_t ring = lds0 + (uint32_t)wave * RS * STEP;
+
+  // per-lane byte offsets of the loads of one step, relative to the step's first element of A / B; a load
+  // carries the instruction offset (j & 3) * 1024 (see Operand::init), OOB_OFFSET where nothing is to be read
+  uint32_t voa[NA], vob[NB];
+#pragma unroll
+  for (int j = 0; j < NA; ++j) {
+    const uint32_t row = 8 * j + (lane >> 3), c = (lane & 7) ^ swz_k(row);
+    voa[j] = row * (uint32_t)p.lda * 2 + c * 16 - (j & 3) * 1024;
+    if ((int)row >= p.M) voa[j] = OOB_OFFSET;
+  }
+#pragma unroll
+  for (int j = 0; j < NB; ++j) {
+    const uint32_t r = 8 * j + (lane >> 3);  // k-row of the step ([K,N]) or column of the strip ([N,K])
+    if constexpr (BKM) {
+      const uint32_t c = (lane & 7) ^ swz_k(r);
+      vob[j] = r * (uint32_t)p.ldb * 2 + c * 16 - (j & 3) * 1024;
+      if (n0 + (int)r >= p.N) vob[j] = OOB_OFFSET;
+    } else {
+      const uint32_t c = (lane & 7) ^ swz_mn64(r & 31);
+      vob[j] = r * (uint32_t)p.ldb * 2 + c * 16 - (j & 3) * 1024;
+      if (n0 + (int)c * 8 >= p.N) vob[j] = OOB_OFFSET;
+    }
+  }
+  auto rsrc = [](uint64_t base) {
+    i32x4 r;
+    r[0] = (int)(uint32_t)base;
+    r[1] = (int)(uint32_t)(base >> 32);
+    r[2] = (int)0x80000000u;
+    r[3] = 0x00020000;
+    return r;
+  };
+  // all loads of step s of this wave into ring slot `slot`; past K everything is masked (the loads are
+  // still issued, as zero fills, so that the count of loads in flight does not depend on K)
+  auto issue_step = [&](int s, int slot) {
+    const int krem = p.K - s * KTILE;  // depth left from this step on (<= 0: nothing)
+    const uint32_t dst = ring + (uint32_t)slot * STEP;
+    const i32x4 ra = rsrc((uint64_t)p.A + (uint64_t)s * KTILE * 2);
+    const i32x4 rb = rsrc((uint64_t)p.B + (BKM ? ((uint64_t)n0 * p.ldb + (uint64_t)s * KTILE) * 2
+                                                : ((uint64_t)s * KTILE * p.ldb + n0) * 2));
+    static_for<NA>([&](auto jc) {
+      constexpr int j = decltype(jc)::value;
+      uint32_t v = voa[j];
+      const uint32_t c = (lane & 7) ^ swz_k(8 * j + (lane >> 3));
+      if ((int)c * 8 >= krem) v = OOB_OFFSET;
+      if constexpr (j % 4 == 0) dma_set_m0(dst + (j / 4) * 4096);
+      dma16<(j & 3) * 1024>(ra, v);
+    });
+    static_for<NB>([&](auto jc) {
+      constexpr int j = decltype(jc)::value;
+      uint32_t v = vob[j];
+      const uint32_t r = 8 * j + (lane >> 3);
+      if constexpr (BKM) {
+        const uint32_t c = (lane & 7) ^ swz_k(r);
+        if ((int)c * 8 >= krem) v = OOB_OFFSET;
+      } else {
+        if ((int)r >= krem) v = OOB_OFFSET;
+      }
+      if constexpr (j % 4 == 0) dma_set_m0(dst + A_STEP + (j / 4) * 4096);
+      dma16<(j & 3) * 1024>(rb, v);
+    });
+  };
+
+  f32x4 acc[TMF][4];
+#pragma unroll
+  for (int t = 0; t < TMF; ++t)
+#pragma unroll
+    for (int f = 0; f < 4; ++f)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) acc[t][f][v] = 0.f;
+
+  // fragment addresses within a step image (see FragReader)
+  const uint32_t frow = lane & 15, fq = (uint32_t)lane >> 4;
+  uint32_t a_off[2], b_off[2];
+#pragma unroll
+  for (int sl = 0; sl < 2; ++sl) {
+    a_off[sl] = frow * 128 + (((4 * sl + fq) ^ swz_k(frow)) << 4);
+    b_off[sl] = A_STEP + a_off[sl];  // B [N,K]: the same image shape, 64 rows
+  }
+  const uint32_t tr_r = frow >> 2, tr_c = frow & 3, kk = 8 * fq + tr_r;  // B [K,N]: k-row within a slab, the second read adds 4
+
+#pragma unroll
+  for (int r = 0; r < RS; ++r) issue_step(wave + 4 * r, r);
+  int slot = 0;
+  for (int s = wave; s < nsteps; s += 4) {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((RS - 1) * LP) : "memory");
+    const uint32_t img = ring + (uint32_t)slot * STEP;
+    bf16x8 af[2][TMF], bf[2][4];
+#pragma unroll
+    for (int sl = 0; sl < 2; ++sl) {
+#pragma unroll
+      for (int t = 0; t < TMF; ++t) af[sl][t] = lds_read_b128(img + a_off[sl] + t * 2048);
+#pragma unroll
+      for (int f = 0; f < 4; ++f) {
+        if constexpr (BKM) {
+          bf[sl][f] = lds_read_b128(img + b_off[sl] + f * 2048);
+        } else {
+          const uint32_t chunk = (2 * f + (tr_c >> 1)) ^ swz_mn64(kk);
+          const uint32_t ad = img + A_STEP + (32 * sl + kk) * 128 + (chunk << 4) + ((tr_c & 1) << 3);
+          const i16x4 lo = lds_read_tr16(ad), hi = lds_read_tr16(ad + 4 * 128);
+          bf[sl][f] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+        }
+      }
+    }
+    // the fragments must be in registers before the next loads overwrite this slot
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    issue_step(s + 4 * RS, slot);
+    slot = slot + 1 == RS ? 0 : slot + 1;
+#pragma unroll
+    for (int sl = 0; sl < 2; ++sl)
+#pragma unroll
+      for (int t = 0; t < TMF; ++t)
+#pragma unroll
+        for (int f = 0; f < 4; ++f)
+          // B fragment first: a lane ends up with 4 consecutive n of one output row (see gemm_tile_kernel)
+          acc[t][f] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bf[sl][f], af[sl][t], acc[t][f], 0, 0, 0);
+  }
+  // drain the loads still in flight (zero fills past K included) before the rings become the reduction buffer
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  // partial sums of the four waves -> LDS; wave w then sums and writes fragment column w, in wave order
+  NEOGEMM_AS3 f32x4* red = (NEOGEMM_AS3 f32x4*)smem;
+#pragma unroll
+  for (int t = 0; t < TMF; ++t)
+#pragma unroll
+    for (int f = 0; f < 4; ++f) red[((wave * TMF + t) * 4 + f) * 64 + lane] = acc[t][f];
+  __syncthreads();
+  const int col = n0 + 16 * wave + 4 * (int)fq;
+#pragma unroll
+  for (int t = 0; t < TMF; ++t) {
+    f32x4 sum = red[((0 * TMF + t) * 4 + wave) * 64 + lane];
+#pragma unroll
+    for (int w = 1; w < 4; ++w) {
+      const f32x4 v = red[((w * TMF + t) * 4 + wave) * 64 + lane];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) sum[r] += v[r];
+    }
+    const int row = 16 * t + (int)frow;
+    if (row >= p.M || col >= p.N) continue;
+    char* crow = p.C + ((size_t)row * p.ldc + col) * 2;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) sum[r] *= p.alpha;
+    if (p.beta != 0.f) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (col + r < p.N) sum[r] = __builtin_fmaf(p.beta, (float)((const __bf16*)crow)[r], sum[r]);
+    }
+    const bf16x4 o = {(__bf16)sum[0], (__bf16)sum[1], (__bf16)sum[2], (__bf16)sum[3]};
+    if (col + 3 < p.N) {
+      *(bf16x4*)crow = o;
+    } else {
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (col + r < p.N) ((__bf16*)crow)[r] = o[r];
+    }
+  }
+}
+
 // Sum the split-K partials in split order (deterministic) and round once to bf16.
 // Then C = alpha * sum + beta * C.
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ ws, char* C, int M, int N,
@@ -831,6 +1025,7 @@ struct VariantInfo {
 };
 static const VariantInfo kVariants[NEOGEMM_VARIANT_COUNT] = {
     {0, 0, 0}, {16, 16, 4}, {256, 256, 8}, {256, 256, 4}, {128, 128, 4}, {256, 128, 8}, {128, 256, 8}, {64, 128, 4}, {128, 128, 4},
+    {16, 64, 4}, {32, 64, 4}, {64, 64, 4},
 };
 
 template <int BM, int BN, int WGM, int WGN>
@@ -935,6 +1130,22 @@ static void plan_model(int64_t M, int64_t N, int64_t K, bool aligned, int c_layo
         bv = c.variant;
         bs = sp;
       }
+    }
+  }
+  // the skinny-M streaming kernel (row-major C only): one strip of 64 columns and all of K per workgroup, 128 KiB
+  // (M <= 16), 96 KiB (M <= 32) or 64 KiB (M <= 64) of B in flight each at ~2.5 us per round trip; no split-K,
+  // one launch
+  if (c_layout == NEOGEMM_C_ROW && rows <= 64 && batch == 1 && K >= 4 * KTILE) {
+    const double wgs = (double)ceil_div(cols, 64), full = __builtin_floor(wgs / cus), frac = wgs / cus - full;
+    const double rounds = full + (frac > 0.0 ? 0.7 + 0.3 * frac : 0.0);
+    const double wg_us = ((double)K * 128.0 + (double)rows * K * 2.0) / (rows <= 16 ? 51.0e3 : rows <= 32 ? 43.0e3 : 39.0e3);
+    double t = rounds * wg_us;
+    if (t < stream_us) t = stream_us;
+    t += 3.0;
+    if (t < best) {
+      best = t;
+      bv = rows <= 16 ? NEOGEMM_VARIANT_SKINNY16 : rows <= 32 ? NEOGEMM_VARIANT_SKINNY32 : NEOGEMM_VARIANT_SKINNY64;
+      bs = 1;
     }
   }
   *variant = bv;
@@ -1053,6 +1264,48 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
   }
 
   if (!aligned) return NEOGEMM_ERR_UNSUPPORTED;
+
+  if (v == NEOGEMM_VARIANT_SKINNY16 || v == NEOGEMM_VARIANT_SKINNY32 || v == NEOGEMM_VARIANT_SKINNY64) {
+    // what the skinny kernel assumes: row-major C, M within its rows, ld >= 64 for the biased lane offsets
+    // (see Operand::init), whole 16-byte chunks of B [K,N] inside the matrix, one problem
+    const bool ok = c_layout == NEOGEMM_C_ROW && bt.count == 1 && M <= kVariants[v].bm && lda >= 64 && ldb >= 64 &&
+                    (b_layout == NEOGEMM_B_NK || (N & 7) == 0) && (split_k <= 1 || variant == NEOGEMM_VARIANT_AUTO) &&
+                    ceil_div(N, 64) <= 0x7fffffff && !prof;
+    if (!ok) {
+      if (variant != NEOGEMM_VARIANT_AUTO) return NEOGEMM_ERR_UNSUPPORTED;
+      // the 128x128 tile needs the least of the tile kernels, then the generic kernel
+      int st2 = run(A, B, C, M, N, K, lda, ldb, ldc, b_layout, c_layout, workspace, workspace_bytes, hip_stream,
+                    NEOGEMM_VARIANT_T128x128_W4, 1, 0, nullptr, alpha, beta, bt);
+      if (st2 == NEOGEMM_ERR_UNSUPPORTED)
+        st2 = run(A, B, C, M, N, K, lda, ldb, ldc, b_layout, c_layout, workspace, workspace_bytes, hip_stream,
+                  NEOGEMM_VARIANT_GENERIC, 1, 0, nullptr, alpha, beta, bt);
+      return st2;
+    }
+    SkinnyArgs sa{(const char*)A, (const char*)B, (char*)C, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, alpha, beta};
+    const bool bkm = b_layout == NEOGEMM_B_NK;
+    auto go = [&](auto kern, size_t lds) -> hipError_t {
+      static bool attr_done = false;  // per instantiation
+      if (!attr_done) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        attr_done = true;
+      }
+      kern<<<dim3(ceil_div(N, 64)), 256, lds, st>>>(sa);
+      return hipGetLastError();
+    };
+    hipError_t e;
+    if (v == NEOGEMM_VARIANT_SKINNY16)
+      e = bkm ? go(gemm_skinny_kernel<1, 4, true>, 4 * 4 * (2048 + 8192)) : go(gemm_skinny_kernel<1, 4, false>, 4 * 4 * (2048 + 8192));
+    else if (v == NEOGEMM_VARIANT_SKINNY32)
+      e = bkm ? go(gemm_skinny_kernel<2, 3, true>, 4 * 3 * (4096 + 8192)) : go(gemm_skinny_kernel<2, 3, false>, 4 * 3 * (4096 + 8192));
+    else
+      e = bkm ? go(gemm_skinny_kernel<4, 2, true>, 4 * 2 * (8192 + 8192)) : go(gemm_skinny_kernel<4, 2, false>, 4 * 2 * (8192 + 8192));
+    if (e != hipSuccess) {
+      fprintf(stderr, "neogemm: skinny kernel launch failed (variant %d): %s\n", v, hipGetErrorString(e));
+      return NEOGEMM_ERR_LAUNCH;
+    }
+    return NEOGEMM_OK;
+  }
 
   // The tile kernels write row-major output.  Column-major C is the row-major transpose, i.e. the
   // product with the operands' roles exchanged.
