@@ -506,15 +506,14 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
   using T = std::true_type;
   using F = std::false_type;
 
-  // One iteration j of the rotated loop is: sync, second half of slab j, first half of slab j+1.
+  // One iteration j of the main loop is: sync, then the MFMAs of slab j while the fragments of slab j+1 are read.
   // After the sync every wave holds all fragments of slab j in registers and slab j+1 has landed, so
   //   an MN-major slab image j & 3 is dead and takes slab j+4;
   //   for odd j the K-major tile image (j >> 1) % U (U images) is dead and takes tile (j >> 1) + U.
-  // Steady state, period t (iterations j = 2t+1 and 2t+2), what is issued and what each sync keeps in
-  // flight (loads complete in issue order):
+  // Steady state, period t (iterations j = 2t+1 and 2t+2; P0, P1 are the halves of the first, P2, P3 of the
+  // second), what is issued and what each sync keeps in flight (loads complete in issue order):
   //   one K-major operand X (three images), the other Y MN-major:
-  //     P0 = second half of slab 2t+1: first half of X tile t+3      P1 = first half of slab 2t+2: the rest
-  //     P2 = second half of slab 2t+2: Y slab 2t+5                   P3 = first half of slab 2t+3: Y slab 2t+6
+  //     P0: first half of X tile t+3      P1: the rest of it      P2: Y slab 2t+5      P3: Y slab 2t+6
   //     the sync before P0 needs X tile t+1 and Y slab 2t+2: all but the loads of the period before
   //     the sync before P2 needs Y slab 2t+3: all but Y slab 2t+4 and X tile t+3
   //   both K-major (A three images, B two): P0: B tile t+2, P1..P3: A tile t+3
