@@ -559,13 +559,14 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
   slow_iteration(P0{}, std::integral_constant<int, KEEP_PRO>{}, 0);  // nothing was issued since the prologue's wait
 
   int j = 1;
-  // steady: two periods per trip (the MN-major slab images repeat every four slabs, the K-major
-  // tile images rotate at run time); every unit loaded here exists and is full
+  // steady: four periods per trip (the MN-major slab images repeat every four slabs, the K-major tile
+  // images rotate at run time; two periods would do, four halve the cost of the loop branch: +0.5 %);
+  // every unit loaded here exists and is full
   uint32_t x_ld = 0, x_rd = 1;  // of three tile images: the one that takes tile t+3 (= image of tile t) / that holds tile t+1
-  for (; (j >> 1) + 4 < ntile - 1; j += 4) {
+  for (; (j >> 1) + 6 < ntile - 1; j += 8) {
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      // period t = (j >> 1) + u, t & 1 == u since j == 1 (mod 4)
+    for (int u = 0; u < 4; ++u) {
+      // period t = (j >> 1) + u, t & 1 == (u & 1) since j == 1 (mod 8)
       const int jo = j + 2 * u;  // the odd slab 2t+1
       // image index for loads in the first / second half of the period and for reads of slabs 2t+2 / 2t+3:
       //   four slab images: slabs 2t+5, 2t+6 go to (2t+1) & 3, (2t+2) & 3
