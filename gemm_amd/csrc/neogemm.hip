@@ -743,7 +743,7 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// Skinny M (decode shapes: M <= 16 * TMF, row-major C): bound by streaming B from HBM once, so what
+// Skinny M (decode shapes: M <= 16 * TMF; C row-major or, CCOL, column-major): bound by streaming B from HBM once, so what
 // counts is bytes in flight per CU, not MFMA rate.  A workgroup owns a strip of 64 columns of C and the
 // whole of K; no split-K, no second launch.  Its four waves split K between them in steps of 64,
 // each with a private ring of RS steps in LDS that only it fills and reads:
@@ -766,7 +766,7 @@ struct SkinnyArgs {
   long lda, ldb, ldc;
   float alpha, beta;
 };
-template <int TMF, int RS, bool BKM>
+template <int TMF, int RS, bool BKM, bool CCOL = false>
 __global__ __launch_bounds__(256) void gemm_skinny_kernel(SkinnyArgs p) {
   constexpr int BM = 16 * TMF;
   constexpr uint32_t A_STEP = BM * 128, B_STEP = 64 * 128, STEP = A_STEP + B_STEP;
@@ -898,8 +898,10 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(SkinnyArgs p) {
       for (int t = 0; t < TMF; ++t)
 #pragma unroll
         for (int f = 0; f < 4; ++f)
-          // B fragment first: a lane ends up with 4 consecutive n of one output row (see gemm_tile_kernel)
-          acc[t][f] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bf[sl][f], af[sl][t], acc[t][f], 0, 0, 0);
+          // B fragment first: a lane ends up with 4 consecutive n of one output row (see gemm_tile_kernel);
+          // for a column-major C the other way round: 4 consecutive m of one output column
+          if constexpr (CCOL) acc[t][f] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[sl][t], bf[sl][f], acc[t][f], 0, 0, 0);
+          else acc[t][f] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bf[sl][f], af[sl][t], acc[t][f], 0, 0, 0);
   }
   // drain the loads still in flight (zero fills past K included) before the rings become the reduction buffer
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -911,7 +913,6 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(SkinnyArgs p) {
 #pragma unroll
     for (int f = 0; f < 4; ++f) red[((wave * TMF + t) * 4 + f) * 64 + lane] = acc[t][f];
   __syncthreads();
-  const int col = n0 + 16 * wave + 4 * (int)fq;
 #pragma unroll
   for (int t = 0; t < TMF; ++t) {
     f32x4 sum = red[((0 * TMF + t) * 4 + wave) * 64 + lane];
@@ -921,23 +922,26 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(SkinnyArgs p) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) sum[r] += v[r];
     }
-    const int row = 16 * t + (int)frow;
+    // the lane's four elements are consecutive along `fast` (n for a row-major C, m for a column-major one)
+    const int row = CCOL ? 16 * t + 4 * (int)fq : 16 * t + (int)frow;
+    const int col = CCOL ? n0 + 16 * wave + (int)frow : n0 + 16 * wave + 4 * (int)fq;
     if (row >= p.M || col >= p.N) continue;
-    char* crow = p.C + ((size_t)row * p.ldc + col) * 2;
+    const int fast = CCOL ? row : col, fast_end = CCOL ? p.M : p.N;
+    char* cp = p.C + (CCOL ? (size_t)col * p.ldc + row : (size_t)row * p.ldc + col) * 2;
 #pragma unroll
     for (int r = 0; r < 4; ++r) sum[r] *= p.alpha;
     if (p.beta != 0.f) {
 #pragma unroll
       for (int r = 0; r < 4; ++r)
-        if (col + r < p.N) sum[r] = __builtin_fmaf(p.beta, (float)((const __bf16*)crow)[r], sum[r]);
+        if (fast + r < fast_end) sum[r] = __builtin_fmaf(p.beta, (float)((const __bf16*)cp)[r], sum[r]);
     }
     const bf16x4 o = {(__bf16)sum[0], (__bf16)sum[1], (__bf16)sum[2], (__bf16)sum[3]};
-    if (col + 3 < p.N) {
-      *(bf16x4*)crow = o;
+    if (fast + 3 < fast_end) {
+      *(bf16x4*)cp = o;
     } else {
 #pragma unroll
       for (int r = 0; r < 4; ++r)
-        if (col + r < p.N) ((__bf16*)crow)[r] = o[r];
+        if (fast + r < fast_end) ((__bf16*)cp)[r] = o[r];
     }
   }
 }
@@ -1138,10 +1142,11 @@ static void plan_model(int64_t M, int64_t N, int64_t K, bool aligned, int c_layo
       }
     }
   }
-  // the skinny-M streaming kernel (row-major C only): one strip of 64 columns and all of K per workgroup, 128 KiB
+  // the skinny-M streaming kernel: one strip of 64 columns and all of K per workgroup, 128 KiB
   // (M <= 16), 96 KiB (M <= 32) or 64 KiB (M <= 64) of B in flight each at ~2.5 us per round trip; no split-K,
   // one launch
-  if (c_layout == NEOGEMM_C_ROW && rows <= 64 && batch == 1 && K >= 4 * KTILE) {
+  if (M <= 64 && batch == 1 && K >= 4 * KTILE) {
+    const int64_t rows = M, cols = N;  // the kernel's own terms, whatever the layout of C
     const double wgs = (double)ceil_div(cols, 64), full = __builtin_floor(wgs / cus), frac = wgs / cus - full;
     const double rounds = full + (frac > 0.0 ? 0.7 + 0.3 * frac : 0.0);
     const double wg_us = ((double)K * 128.0 + (double)rows * K * 2.0) / (rows <= 16 ? 51.0e3 : rows <= 32 ? 43.0e3 : 39.0e3);
@@ -1272,9 +1277,9 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
   if (!aligned) return NEOGEMM_ERR_UNSUPPORTED;
 
   if (v == NEOGEMM_VARIANT_SKINNY16 || v == NEOGEMM_VARIANT_SKINNY32 || v == NEOGEMM_VARIANT_SKINNY64) {
-    // what the skinny kernel assumes: row-major C, M within its rows, ld >= 64 for the biased lane offsets
+    // what the skinny kernel assumes: M within its rows, ld >= 64 for the biased lane offsets
     // (see Operand::init), whole 16-byte chunks of B [K,N] inside the matrix, one problem
-    const bool ok = c_layout == NEOGEMM_C_ROW && bt.count == 1 && M <= kVariants[v].bm && lda >= 64 && ldb >= 64 &&
+    const bool ok = bt.count == 1 && M <= kVariants[v].bm && lda >= 64 && ldb >= 64 &&
                     (b_layout == NEOGEMM_B_NK || (N & 7) == 0) && (split_k <= 1 || variant == NEOGEMM_VARIANT_AUTO) &&
                     ceil_div(N, 64) <= 0x7fffffff && !prof;
     if (!ok) {
@@ -1288,7 +1293,7 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
       return st2;
     }
     SkinnyArgs sa{(const char*)A, (const char*)B, (char*)C, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, alpha, beta};
-    const bool bkm = b_layout == NEOGEMM_B_NK;
+    const bool bkm = b_layout == NEOGEMM_B_NK, ccol = c_layout == NEOGEMM_C_COL;
     auto go = [&](auto kern, size_t lds) -> hipError_t {
       static bool attr_done = false;  // per instantiation
       if (!attr_done) {
@@ -1299,13 +1304,17 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
       kern<<<dim3(ceil_div(N, 64)), 256, lds, st>>>(sa);
       return hipGetLastError();
     };
+    auto pick = [&](auto tmf, auto rs) -> hipError_t {
+      constexpr int TMF = decltype(tmf)::value, RS = decltype(rs)::value;
+      constexpr size_t lds = (size_t)4 * RS * (TMF * 2048 + 8192);
+      if (bkm) return ccol ? go(gemm_skinny_kernel<TMF, RS, true, true>, lds) : go(gemm_skinny_kernel<TMF, RS, true, false>, lds);
+      return ccol ? go(gemm_skinny_kernel<TMF, RS, false, true>, lds) : go(gemm_skinny_kernel<TMF, RS, false, false>, lds);
+    };
+    using std::integral_constant;
     hipError_t e;
-    if (v == NEOGEMM_VARIANT_SKINNY16)
-      e = bkm ? go(gemm_skinny_kernel<1, 4, true>, 4 * 4 * (2048 + 8192)) : go(gemm_skinny_kernel<1, 4, false>, 4 * 4 * (2048 + 8192));
-    else if (v == NEOGEMM_VARIANT_SKINNY32)
-      e = bkm ? go(gemm_skinny_kernel<2, 3, true>, 4 * 3 * (4096 + 8192)) : go(gemm_skinny_kernel<2, 3, false>, 4 * 3 * (4096 + 8192));
-    else
-      e = bkm ? go(gemm_skinny_kernel<4, 2, true>, 4 * 2 * (8192 + 8192)) : go(gemm_skinny_kernel<4, 2, false>, 4 * 2 * (8192 + 8192));
+    if (v == NEOGEMM_VARIANT_SKINNY16) e = pick(integral_constant<int, 1>{}, integral_constant<int, 4>{});
+    else if (v == NEOGEMM_VARIANT_SKINNY32) e = pick(integral_constant<int, 2>{}, integral_constant<int, 3>{});
+    else e = pick(integral_constant<int, 4>{}, integral_constant<int, 2>{});
     if (e != hipSuccess) {
       fprintf(stderr, "neogemm: skinny kernel launch failed (variant %d): %s\n", v, hipGetErrorString(e));
       return NEOGEMM_ERR_LAUNCH;
