@@ -34,6 +34,10 @@ typedef __attribute__((ext_vector_type(8))) short i16x8;
 static constexpr int KT = 32;                        // K depth of one MFMA step / one slab (bf16 elements)
 static constexpr int KTILE = 64;                     // K depth of a K-major LDS image, and the split-K unit
 static constexpr uint32_t OOB_OFFSET = 0x80000000u;  // >= every num_records this file builds
+// Load j of a run of four carries the instruction offset (j & 3) * 1024, which moves the global and the LDS
+// address alike; the lane offsets are lowered by it and raised by VOFF_BIAS (so that they cannot go negative,
+// whatever the leading dimension), and the resource base is lowered by VOFF_BIAS in turn.
+static constexpr uint32_t VOFF_BIAS = 3 * 1024;
 
 // ---------------------------------------------------------------------------------------------
 // LDS images and their swizzles.  K is consumed in slabs of 32 (one v_mfma_f32_16x16x32_bf16 step).
@@ -147,9 +151,7 @@ struct Operand {
   // Every lane offset that would leave the matrix is replaced by OOB_OFFSET, which the buffer range
   // check (num_records = 2 GiB, constant) turns into a zero fill without a memory access; all other
   // offsets address bytes inside the matrix, so the resource needs no exact size and only its base
-  // moves along K.  Load j carries the instruction offset (j & 3) * 1024, which moves the global and the
-  // LDS address alike: the lane offsets are biased by it (rows grow faster than the bias, see the host
-  // checks on ld).
+  // moves along K.  (See VOFF_BIAS for the instruction offsets.)
   __device__ __forceinline__ void init(const char* ptr, long ld, int rows_total, int r0, int k_begin, int wave,
                                        int lane) {
     if constexpr (KMAJOR) {
@@ -159,7 +161,7 @@ struct Operand {
       for (int j = 0; j < IPW; ++j) {
         uint32_t row = (wave * IPW + j) * 8 + (lane >> 3);
         uint32_t c = (lane & 7) ^ swz_k(row);
-        voff[j] = row * (uint32_t)ld * 2 + c * 16 - (j & 3) * 1024;  // row >= 8*j and ld >= 64 keep this >= 0
+        voff[j] = row * (uint32_t)ld * 2 + c * 16 + VOFF_BIAS - (j & 3) * 1024;
         if (r0 + (int)row >= rows_total) voff[j] = OOB_OFFSET;
       }
     } else {
@@ -169,7 +171,7 @@ struct Operand {
       for (int j = 0; j < IPW; ++j) {
         uint32_t krow = (wave * IPW + j) * KR + lane / CPR;
         uint32_t c = (lane % CPR) ^ swz_mn(krow);
-        voff[j] = krow * (uint32_t)ld * 2 + c * 16 - (j & 3) * 1024;  // krow >= KR*j and ld >= ROWS keep this >= 0
+        voff[j] = krow * (uint32_t)ld * 2 + c * 16 + VOFF_BIAS - (j & 3) * 1024;
         // a chunk past the last column would wrap into the next k-row (rows_total % 8 == 0: no straddling)
         if (r0 + (int)c * 8 >= rows_total) voff[j] = OOB_OFFSET;
       }
@@ -196,8 +198,9 @@ struct Operand {
 
   __device__ __forceinline__ i32x4 rsrc() const {
     i32x4 r;
-    r[0] = (int)(uint32_t)base;
-    r[1] = (int)(uint32_t)(base >> 32);  // a 48-bit address: bits 16.. (stride, swizzle) stay 0
+    const uint64_t b = base - VOFF_BIAS;
+    r[0] = (int)(uint32_t)b;
+    r[1] = (int)(uint32_t)(b >> 32);  // a 48-bit address: bits 16.. (stride, swizzle) stay 0
     r[2] = (int)0x80000000u;
     r[3] = 0x00020000;
     return r;
@@ -786,7 +789,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(SkinnyArgs p) {
 #pragma unroll
   for (int j = 0; j < NA; ++j) {
     const uint32_t row = 8 * j + (lane >> 3), c = (lane & 7) ^ swz_k(row);
-    voa[j] = row * (uint32_t)p.lda * 2 + c * 16 - (j & 3) * 1024;
+    voa[j] = row * (uint32_t)p.lda * 2 + c * 16 + VOFF_BIAS - (j & 3) * 1024;
     if ((int)row >= p.M) voa[j] = OOB_OFFSET;
   }
 #pragma unroll
@@ -794,11 +797,11 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(SkinnyArgs p) {
     const uint32_t r = 8 * j + (lane >> 3);  // k-row of the step ([K,N]) or column of the strip ([N,K])
     if constexpr (BKM) {
       const uint32_t c = (lane & 7) ^ swz_k(r);
-      vob[j] = r * (uint32_t)p.ldb * 2 + c * 16 - (j & 3) * 1024;
+      vob[j] = r * (uint32_t)p.ldb * 2 + c * 16 + VOFF_BIAS - (j & 3) * 1024;
       if (n0 + (int)r >= p.N) vob[j] = OOB_OFFSET;
     } else {
       const uint32_t c = (lane & 7) ^ swz_mn64(r & 31);
-      vob[j] = r * (uint32_t)p.ldb * 2 + c * 16 - (j & 3) * 1024;
+      vob[j] = r * (uint32_t)p.ldb * 2 + c * 16 + VOFF_BIAS - (j & 3) * 1024;
       if (n0 + (int)c * 8 >= p.N) vob[j] = OOB_OFFSET;
     }
   }
@@ -810,6 +813,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(SkinnyArgs p) {
   const int s_end = BKM ? (s_begin + qsteps < nsteps ? s_begin + qsteps : nsteps) : nsteps;
   auto rsrc = [](uint64_t base) {
     i32x4 r;
+    base -= VOFF_BIAS;
     r[0] = (int)(uint32_t)base;
     r[1] = (int)(uint32_t)(base >> 32);
     r[2] = (int)0x80000000u;
@@ -1277,9 +1281,9 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
   if (!aligned) return NEOGEMM_ERR_UNSUPPORTED;
 
   if (v == NEOGEMM_VARIANT_SKINNY16 || v == NEOGEMM_VARIANT_SKINNY32 || v == NEOGEMM_VARIANT_SKINNY64) {
-    // what the skinny kernel assumes: M within its rows, ld >= 64 for the biased lane offsets
-    // (see Operand::init), whole 16-byte chunks of B [K,N] inside the matrix, one problem
-    const bool ok = bt.count == 1 && M <= kVariants[v].bm && lda >= 64 && ldb >= 64 &&
+    // what the skinny kernel assumes: M within its rows, whole 16-byte chunks of B [K,N] inside the matrix,
+    // one problem
+    const bool ok = bt.count == 1 && M <= kVariants[v].bm &&
                     (b_layout == NEOGEMM_B_NK || (N & 7) == 0) && (split_k <= 1 || variant == NEOGEMM_VARIANT_AUTO) &&
                     ceil_div(N, 64) <= 0x7fffffff && !prof;
     if (!ok) {
@@ -1339,12 +1343,9 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
   a.batch = (int)bt.count;
   a.K = (int)K;
   const VariantInfo& vi = kVariants[v];
-  // What the tile kernels assume about an operand (see Operand::init): an MN-major tile needs >= 128
-  // rows for its swizzle, ld >= tile rows and a row count that is a multiple of 8 (16-byte chunks must
-  // not straddle the matrix edge), a K-major one ld >= 64, so that the per-lane offsets, which are
-  // biased by the instruction offsets of the loads, stay non-negative.
-  const bool fits = (ak ? a.lda >= 64 : (vi.bm >= 128 && a.lda >= vi.bm && (a.M & 7) == 0)) &&
-                    (bk ? a.ldb >= 64 : (vi.bn >= 128 && a.ldb >= vi.bn && (a.N & 7) == 0));
+  // What the tile kernels assume about an MN-major operand (see Operand::init): a tile of >= 128 rows for
+  // its swizzle and a row count that is a multiple of 8 (16-byte chunks must not straddle the matrix edge).
+  const bool fits = (ak || (vi.bm >= 128 && (a.M & 7) == 0)) && (bk || (vi.bn >= 128 && (a.N & 7) == 0));
   if (!fits) {
     if (variant != NEOGEMM_VARIANT_AUTO) return NEOGEMM_ERR_UNSUPPORTED;
     // the planned tile is too wide for an MN-major operand: the 128x128 tile needs the least, then generic

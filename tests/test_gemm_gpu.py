@@ -39,7 +39,7 @@ def run_abi(A, B, dev, b_layout=g.B_KN, c_layout=g.C_ROW, variant=None, split_k=
     except g.NeoGemmError as e:
         if e.status == _abi.ERR_UNSUPPORTED and variant not in (None, g.VARIANT_GENERIC) and not strict:
             # a forced tile variant may refuse a layout (an MN-major operand needs a tile >= 128 wide, ld >= tile,
-            # rows % 8 == 0; a K-major one ld >= 64): refusing is the documented behaviour, mis-running would not be
+            # rows % 8 == 0): refusing is the documented behaviour, mis-running would not be
             pytest.skip(f"variant {variant} refuses this layout/shape (status {e.status})")
         raise
     torch.cuda.synchronize()
@@ -89,8 +89,6 @@ def test_ones(dev, K):
     B = torch.ones(K, 264, dtype=torch.bfloat16)
     want = torch.tensor(float(K)).to(torch.bfloat16)   # 264 -> 264, 1000 -> 1000, exact sums then RNE
     for variant in (None, g.VARIANT_T128x128_W4, g.VARIANT_T256x256_W4):
-        if variant is not None and K < 32:
-            continue   # the tile kernels need ld >= 32; the library's own choice covers such shapes
         assert torch.all(run_abi(A, B, dev, variant=variant) == want)
 
 
@@ -203,9 +201,8 @@ def test_ragged_shapes_forced_tile_kernels(dev, variant, M, N, K):
         try:
             got = run_abi(A, B, dev, b_layout, g.C_ROW, variant, strict=True)
         except g.NeoGemmError as e:
-            # an MN-major tile narrower than its image, N % 8 != 0, or a K-major leading dimension
-            # below the 64-deep LDS tile is refused, never mis-run
-            assert e.status == _abi.ERR_UNSUPPORTED and (b_layout == g.B_KN or K < 64)
+            # an MN-major operand on a tile below 128 rows, or N % 8 != 0, is refused, never mis-run
+            assert e.status == _abi.ERR_UNSUPPORTED and b_layout == g.B_KN
             continue
         o.assert_parity(got, A, Bkn, what=f"{M}x{N}x{K} v{variant} b{b_layout}")
 
@@ -590,3 +587,18 @@ def test_skinny_known_answers_and_refusals(dev):
         got = run_scaled(A, Bkn, C0, dev, 1.5, -0.5, g.B_KN, c_layout)
         ulp, fro = o.scaled_parity(got, A, Bkn, C0, 1.5, -0.5)
         assert ulp <= 1.0 and fro <= 1e-3
+
+
+def test_narrow_operands_run_the_tile_kernels(dev):
+    """Leading dimensions below the tile width (N < 128 with B [K,N], K < 64) stay on the MFMA path."""
+    for (M, N, K) in ((1024, 16, 512), (2048, 64, 4096), (300, 96, 200), (512, 512, 8), (512, 40, 24), (8, 8, 32),
+                      (14336, 16, 4096)):
+        assert g.plan(M, N, K)[0] != g.VARIANT_GENERIC
+        A, Bkn = o.make_inputs(M, N, K, seed=N + K)
+        for b_layout in (g.B_KN, g.B_NK):
+            for c_layout in (g.C_ROW, g.C_COL):
+                got = run_abi(A, layouts(Bkn, b_layout), dev, b_layout, c_layout)
+                o.assert_parity(got, A, Bkn, what=f"{M}x{N}x{K} b{b_layout} c{c_layout}")
+        for variant in (g.VARIANT_T128x128_W4, g.VARIANT_T256x256_W4):
+            got = run_abi(A, Bkn, dev, g.B_KN, g.C_ROW, variant, strict=True)
+            o.assert_parity(got, A, Bkn, what=f"{M}x{N}x{K} v{variant}")
