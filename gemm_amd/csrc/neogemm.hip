@@ -1103,7 +1103,7 @@ static const PlanCand kPlanCands[] = {
     {NEOGEMM_VARIANT_T64x128_W4, 0.35, 2.5, 1.0, 2},
 };
 static void plan_model(int64_t M, int64_t N, int64_t K, bool aligned, int c_layout, int* variant, int* split_k,
-                       int64_t batch = 1) {
+                       int64_t batch = 1, int b_layout = NEOGEMM_B_KN) {
   if (!aligned || K == 0) {
     *variant = NEOGEMM_VARIANT_GENERIC;
     *split_k = 1;
@@ -1149,8 +1149,10 @@ static void plan_model(int64_t M, int64_t N, int64_t K, bool aligned, int c_layo
   // the skinny-M streaming kernel: one strip of 64 columns and all of K per workgroup, 128 KiB
   // (M <= 16), 96 KiB (M <= 32) or 64 KiB (M <= 64) of B in flight each at ~2.5 us per round trip; no split-K,
   // one launch
-  if (M <= 64 && batch == 1 && K >= 4 * KTILE) {
-    const int64_t rows = M, cols = N;  // the kernel's own terms, whatever the layout of C
+  // With B [N,K] and N <= 64 < M the same kernel runs the transposed problem (the wide operand is A then).
+  const bool skinny_m = M <= 64, skinny_n = !skinny_m && N <= 64 && b_layout == NEOGEMM_B_NK;
+  if ((skinny_m || skinny_n) && batch == 1 && K >= 4 * KTILE) {
+    const int64_t rows = skinny_m ? M : N, cols = skinny_m ? N : M;  // the kernel's own terms, whatever the layout of C
     const double wgs = (double)ceil_div(cols, 64), full = __builtin_floor(wgs / cus), frac = wgs / cus - full;
     const double rounds = full + (frac > 0.0 ? 0.7 + 0.3 * frac : 0.0);
     const double wg_us = ((double)K * 128.0 + (double)rows * K * 2.0) / (rows <= 16 ? 51.0e3 : rows <= 32 ? 43.0e3 : 39.0e3);
@@ -1213,7 +1215,7 @@ static const std::vector<PlanEntry>& plan_table() {
   return table;
 }
 static void plan(int64_t M, int64_t N, int64_t K, bool aligned, int c_layout, int* variant, int* split_k,
-                 int64_t batch = 1) {
+                 int64_t batch = 1, int b_layout = NEOGEMM_B_KN) {
   if (aligned && K > 0 && batch == 1) {
     for (const PlanEntry& e : plan_table())
       if (e.M == M && e.N == N && e.K == K && e.c_layout == c_layout) {
@@ -1222,7 +1224,7 @@ static void plan(int64_t M, int64_t N, int64_t K, bool aligned, int c_layout, in
         return;
       }
   }
-  plan_model(M, N, K, aligned, c_layout, variant, split_k, batch);
+  plan_model(M, N, K, aligned, c_layout, variant, split_k, batch, b_layout);
 }
 
 // A batch of `count` problems of one shape; strides in elements between consecutive problems (0: shared operand).
@@ -1257,7 +1259,7 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
   int v = variant, s = split_k;
   if (v == NEOGEMM_VARIANT_AUTO) {
     int pv, ps;
-    plan(M, N, K, aligned, c_layout, &pv, &ps, bt.count);
+    plan(M, N, K, aligned, c_layout, &pv, &ps, bt.count, b_layout);
     v = pv;
     if (s == 0) s = ps;
   }
@@ -1282,10 +1284,11 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
 
   if (v == NEOGEMM_VARIANT_SKINNY16 || v == NEOGEMM_VARIANT_SKINNY32 || v == NEOGEMM_VARIANT_SKINNY64) {
     // what the skinny kernel assumes: M within its rows, whole 16-byte chunks of B [K,N] inside the matrix,
-    // one problem
-    const bool ok = bt.count == 1 && M <= kVariants[v].bm &&
-                    (b_layout == NEOGEMM_B_NK || (N & 7) == 0) && (split_k <= 1 || variant == NEOGEMM_VARIANT_AUTO) &&
-                    ceil_div(N, 64) <= 0x7fffffff && !prof;
+    // one problem.  If M is too large but N fits and B is [N,K], it runs the transposed problem
+    // C^T = B * A^T: its small operand is B then, its wide one A, and the layout of C flips.
+    const bool swap = M > kVariants[v].bm && N <= kVariants[v].bm && b_layout == NEOGEMM_B_NK;
+    const bool ok = bt.count == 1 && (M <= kVariants[v].bm || swap) &&
+                    (b_layout == NEOGEMM_B_NK || (N & 7) == 0) && (split_k <= 1 || variant == NEOGEMM_VARIANT_AUTO) && !prof;
     if (!ok) {
       if (variant != NEOGEMM_VARIANT_AUTO) return NEOGEMM_ERR_UNSUPPORTED;
       // the 128x128 tile needs the least of the tile kernels, then the generic kernel
@@ -1297,7 +1300,12 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
       return st2;
     }
     SkinnyArgs sa{(const char*)A, (const char*)B, (char*)C, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, alpha, beta};
-    const bool bkm = b_layout == NEOGEMM_B_NK, ccol = c_layout == NEOGEMM_C_COL;
+    bool bkm = b_layout == NEOGEMM_B_NK, ccol = c_layout == NEOGEMM_C_COL;
+    if (swap) {
+      sa = SkinnyArgs{(const char*)B, (const char*)A, (char*)C, (int)N, (int)M, (int)K, (long)ldb, (long)lda, (long)ldc, alpha, beta};
+      bkm = true;    // A [M,K] takes the place of a B [N,K]
+      ccol = !ccol;  // a row-major C[m][n] is the column-major C^T
+    }
     auto go = [&](auto kern, size_t lds) -> hipError_t {
       static bool attr_done = false;  // per instantiation
       if (!attr_done) {
@@ -1305,7 +1313,7 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
         if (e != hipSuccess) return e;
         attr_done = true;
       }
-      kern<<<dim3(ceil_div(N, 64)), 256, lds, st>>>(sa);
+      kern<<<dim3(ceil_div(sa.N, 64)), 256, lds, st>>>(sa);
       return hipGetLastError();
     };
     auto pick = [&](auto tmf, auto rs) -> hipError_t {
@@ -1482,10 +1490,10 @@ size_t neogemm_bf16_workspace_bytes(int64_t M, int64_t N, int64_t K) {
 
 int neogemm_bf16_plan(int64_t M, int64_t N, int64_t K, int b_layout, int c_layout, int aligned, int* variant,
                       int* split_k) {
-  (void)b_layout;
   if (!variant || !split_k || M < 0 || N < 0 || K < 0) return NEOGEMM_ERR_BAD_ARG;
   if (c_layout != NEOGEMM_C_ROW && c_layout != NEOGEMM_C_COL) return NEOGEMM_ERR_BAD_ARG;
-  neogemm::plan(M, N, K, aligned != 0, c_layout, variant, split_k);
+  if (b_layout != NEOGEMM_B_KN && b_layout != NEOGEMM_B_NK) return NEOGEMM_ERR_BAD_ARG;
+  neogemm::plan(M, N, K, aligned != 0, c_layout, variant, split_k, 1, b_layout);
   return NEOGEMM_OK;
 }
 

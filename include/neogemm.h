@@ -50,7 +50,7 @@ extern "C" {
 #define NEOGEMM_VARIANT_T128x256_W8 6 /* 128x256, 8 wave64 (2x4) */
 #define NEOGEMM_VARIANT_T64x128_W4 7  /* 64x128, 4 wave64 (1x4) */
 #define NEOGEMM_VARIANT_T128x128_W4S 8 /* 128x128, 4 wave64 (1x4) */
-/* Skinny M: a strip of 64 columns and all of K per workgroup, no split-K (decode shapes). */
+/* Skinny M (or, with B [N,K], skinny N): a strip of 64 columns and all of K per workgroup, no split-K (decode shapes). */
 #define NEOGEMM_VARIANT_SKINNY16 9  /* M <= 16 */
 #define NEOGEMM_VARIANT_SKINNY32 10 /* M <= 32 */
 #define NEOGEMM_VARIANT_SKINNY64 11 /* M <= 64 */

@@ -602,3 +602,21 @@ def test_narrow_operands_run_the_tile_kernels(dev):
         for variant in (g.VARIANT_T128x128_W4, g.VARIANT_T256x256_W4):
             got = run_abi(A, Bkn, dev, g.B_KN, g.C_ROW, variant, strict=True)
             o.assert_parity(got, A, Bkn, what=f"{M}x{N}x{K} v{variant}")
+
+
+def test_skinny_n_runs_the_transposed_problem(dev):
+    """N <= 64 < M with B [N,K]: the skinny kernel computes C^T = B * A^T (small operand B, wide operand A)."""
+    assert g.plan(14336, 16, 4096, b_layout=g.B_NK)[0] == g.VARIANT_SKINNY16
+    assert g.plan(14336, 48, 4096, b_layout=g.B_NK, c_layout=g.C_COL)[0] == g.VARIANT_SKINNY64
+    assert g.plan(14336, 16, 4096, b_layout=g.B_KN)[0] not in (g.VARIANT_SKINNY16, g.VARIANT_GENERIC)
+    for variant, cols in SKINNY:
+        for (M, N, K) in ((1000, cols, 520), (4096, cols - 4, 1032), (200, 8, 72), (14336, cols, 512)):
+            A, Bkn = o.make_inputs(M, N, K, seed=M + N)
+            for c_layout in (g.C_ROW, g.C_COL):
+                for v in (variant, None):
+                    got = run_abi(A, layouts(Bkn, g.B_NK), dev, g.B_NK, c_layout, v, strict=True)
+                    o.assert_parity(got, A, Bkn, what=f"skinny-n v{v} {M}x{N}x{K} c{c_layout}")
+        # with B [K,N] the small operand is not K-major: refused when forced
+        A, Bkn = o.make_inputs(512, cols, 256, seed=1)
+        with pytest.raises(g.NeoGemmError):
+            run_abi(A, Bkn, dev, g.B_KN, g.C_ROW, variant, strict=True)
