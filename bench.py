@@ -111,7 +111,7 @@ def main():
                      "frac": round(achieved / PEAK_TFLOPS, 4),
                      # HBM-side bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a plain copy
                      # (profiles/gemm_tile_256x256_w4_8192cubed.txt); the algorithmic figure is 402.7e6
-                     "traffic": 1.768e9,
+                     "traffic": 1.762e9,
                      "kernel_ms": round(ev_ms, 5), "flop_per_launch": flop},
         "parity": {"ok": bool(parity_ok), "rows_checked": 128, **{k: rep[k] for k in ("max_ulp", "max_ulp_floored", "rel_fro")}},
         "vendor": {"lib": "torch.matmul (hipBLASLt/rocBLAS)", "tflops_b_kn": round(flop / vend_ms / 1e9, 2),
