@@ -141,7 +141,8 @@ struct Operand {
   static constexpr int CPR = ROWS / 8;                     // 16-byte chunks per k-row (MN-major)
   static constexpr int KR = 64 / CPR;                      // k-rows per wave-load (MN-major)
   static_assert(NINSTR % NW == 0 && IPW >= 1 && IPW <= 8, "unit loads must divide evenly over the waves");
-  static_assert(KMAJOR || ROWS >= 128, "MN-major swizzle needs >= 16 chunks per k-row");
+  static_assert(KMAJOR || (ROWS >= 128 && (ROWS & (ROWS - 1)) == 0),
+                "MN-major: >= 16 chunks per k-row for the swizzle, a power of two so that a wave-load covers whole k-rows");
 
   uint32_t voff[IPW];
   uint64_t base;
@@ -1039,7 +1040,7 @@ struct VariantInfo {
 };
 static const VariantInfo kVariants[NEOGEMM_VARIANT_COUNT] = {
     {0, 0, 0}, {16, 16, 4}, {256, 256, 8}, {256, 256, 4}, {128, 128, 4}, {256, 128, 8}, {128, 256, 8}, {64, 128, 4}, {128, 128, 4},
-    {16, 64, 4}, {32, 64, 4}, {64, 64, 4},
+    {16, 64, 4}, {32, 64, 4}, {64, 64, 4}, {192, 256, 4},
 };
 
 template <int BM, int BN, int WGM, int WGN>
@@ -1066,10 +1067,10 @@ static hipError_t launch_tile(const TileArgs& a, bool ak, bool bk, hipStream_t s
   }
   if (ak && bk) return go(gemm_tile_kernel<BM, BN, WGM, WGN, true, true>);
   if (ak && !bk) {
-    if constexpr (BN >= 128) return go(gemm_tile_kernel<BM, BN, WGM, WGN, true, false>);
+    if constexpr (BN >= 128 && (BN & (BN - 1)) == 0) return go(gemm_tile_kernel<BM, BN, WGM, WGN, true, false>);
   }
   if (!ak && bk) {
-    if constexpr (BM >= 128) return go(gemm_tile_kernel<BM, BN, WGM, WGN, false, true>);
+    if constexpr (BM >= 128 && (BM & (BM - 1)) == 0) return go(gemm_tile_kernel<BM, BN, WGM, WGN, false, true>);
   }
   return hipErrorInvalidValue;
 }
@@ -1100,7 +1101,7 @@ struct PlanCand {
 static const PlanCand kPlanCands[] = {
     {NEOGEMM_VARIANT_T256x256_W4, 1.33, 9.0, 12.0, 1}, {NEOGEMM_VARIANT_T128x256_W8, 0.78, 6.0, 5.0, 1},
     {NEOGEMM_VARIANT_T256x128_W8, 0.78, 6.0, 5.0, 1},  {NEOGEMM_VARIANT_T128x128_W4, 0.50, 3.0, 2.0, 2},
-    {NEOGEMM_VARIANT_T64x128_W4, 0.35, 2.5, 1.0, 2},
+    {NEOGEMM_VARIANT_T64x128_W4, 0.35, 2.5, 1.0, 2},    {NEOGEMM_VARIANT_T192x256_W4, 1.0, 7.0, 9.0, 1},
 };
 static void plan_model(int64_t M, int64_t N, int64_t K, bool aligned, int c_layout, int* variant, int* split_k,
                        int64_t batch = 1, int b_layout = NEOGEMM_B_KN) {
@@ -1120,6 +1121,8 @@ static void plan_model(int64_t M, int64_t N, int64_t K, bool aligned, int c_layo
   for (const PlanCand& c : kPlanCands) {
     // the 64x128 tile has too little in flight to stream from HBM: only for problems that stay in cache
     if (c.variant == NEOGEMM_VARIANT_T64x128_W4 && bytes > 32e6) continue;
+    // 192 rows only of a K-major operand (an MN-major image needs a power of two)
+    if (c.variant == NEOGEMM_VARIANT_T192x256_W4 && c_layout == NEOGEMM_C_COL && b_layout != NEOGEMM_B_NK) continue;
     const double tiles = (double)ceil_div(rows, kVariants[c.variant].bm) * (double)ceil_div(cols, kVariants[c.variant].bn);
     for (int sp : kSplits) {
       if (sp > 1 && ktiles / sp < 2) break;  // at least 128 deep per split
@@ -1351,9 +1354,11 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
   a.batch = (int)bt.count;
   a.K = (int)K;
   const VariantInfo& vi = kVariants[v];
-  // What the tile kernels assume about an MN-major operand (see Operand::init): a tile of >= 128 rows for
-  // its swizzle and a row count that is a multiple of 8 (16-byte chunks must not straddle the matrix edge).
-  const bool fits = (ak || (vi.bm >= 128 && (a.M & 7) == 0)) && (bk || (vi.bn >= 128 && (a.N & 7) == 0));
+  // What the tile kernels assume about an MN-major operand (see Operand::init): a tile of >= 128 rows, a power
+  // of two, for its swizzle and a row count that is a multiple of 8 (16-byte chunks must not straddle the
+  // matrix edge).
+  auto mn_ok = [](int tile, int rows) { return tile >= 128 && (tile & (tile - 1)) == 0 && (rows & 7) == 0; };
+  const bool fits = (ak || mn_ok(vi.bm, a.M)) && (bk || mn_ok(vi.bn, a.N));
   if (!fits) {
     if (variant != NEOGEMM_VARIANT_AUTO) return NEOGEMM_ERR_UNSUPPORTED;
     // the planned tile is too wide for an MN-major operand: the 128x128 tile needs the least, then generic
@@ -1394,6 +1399,7 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
     case NEOGEMM_VARIANT_T128x256_W8: e = launch_tile<128, 256, 2, 4>(a, ak, bk, st); break;
     case NEOGEMM_VARIANT_T64x128_W4: e = launch_tile<64, 128, 1, 4>(a, ak, bk, st); break;
     case NEOGEMM_VARIANT_T128x128_W4S: e = launch_tile<128, 128, 1, 4>(a, ak, bk, st); break;
+    case NEOGEMM_VARIANT_T192x256_W4: e = launch_tile<192, 256, 2, 2>(a, ak, bk, st); break;
     default: return NEOGEMM_ERR_BAD_ARG;
   }
   if (e != hipSuccess) {

@@ -54,7 +54,10 @@ extern "C" {
 #define NEOGEMM_VARIANT_SKINNY16 9  /* M <= 16 */
 #define NEOGEMM_VARIANT_SKINNY32 10 /* M <= 32 */
 #define NEOGEMM_VARIANT_SKINNY64 11 /* M <= 64 */
-#define NEOGEMM_VARIANT_COUNT 12
+/* 192x256, 4 wave64 (2x2): 3/4 of the 256x256 tile, for tile counts that fill the 256 CUs better (3072, 6144 ...);
+   the operand that supplies the 192 rows must be K-major (A for row-major C; B [N,K] for column-major C). */
+#define NEOGEMM_VARIANT_T192x256_W4 12
+#define NEOGEMM_VARIANT_COUNT 13
 
 /*
  * C = A * op(B), bf16 in, fp32 accumulate, bf16 out.
