@@ -1039,7 +1039,7 @@ struct VariantInfo {
   int bm, bn, nwaves;
 };
 static const VariantInfo kVariants[NEOGEMM_VARIANT_COUNT] = {
-    {0, 0, 0}, {16, 16, 4}, {256, 256, 8}, {256, 256, 4}, {128, 128, 4}, {256, 128, 8}, {128, 256, 8}, {64, 128, 4}, {128, 128, 4},
+    {0, 0, 0}, {16, 16, 4}, {256, 256, 8}, {256, 256, 4}, {128, 128, 4}, {256, 128, 4}, {128, 256, 4}, {64, 128, 4}, {128, 128, 4},
     {16, 64, 4}, {32, 64, 4}, {64, 64, 4}, {192, 256, 4},
 };
 
@@ -1099,8 +1099,8 @@ struct PlanCand {
   int per_cu;
 };
 static const PlanCand kPlanCands[] = {
-    {NEOGEMM_VARIANT_T256x256_W4, 1.33, 9.0, 12.0, 1}, {NEOGEMM_VARIANT_T128x256_W8, 0.78, 6.0, 5.0, 1},
-    {NEOGEMM_VARIANT_T256x128_W8, 0.78, 6.0, 5.0, 1},  {NEOGEMM_VARIANT_T128x128_W4, 0.50, 3.0, 2.0, 2},
+    {NEOGEMM_VARIANT_T256x256_W4, 1.33, 9.0, 12.0, 1}, {NEOGEMM_VARIANT_T128x256_W4, 0.78, 6.0, 5.0, 1},
+    {NEOGEMM_VARIANT_T256x128_W4, 0.78, 6.0, 5.0, 1},  {NEOGEMM_VARIANT_T128x128_W4, 0.50, 3.0, 2.0, 2},
     {NEOGEMM_VARIANT_T64x128_W4, 0.35, 2.5, 1.0, 2},    {NEOGEMM_VARIANT_T192x256_W4, 1.0, 7.0, 9.0, 1},
 };
 static void plan_model(int64_t M, int64_t N, int64_t K, bool aligned, int c_layout, int* variant, int* split_k,
@@ -1395,8 +1395,8 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
     case NEOGEMM_VARIANT_T256x256_W8: e = launch_tile<256, 256, 2, 4>(a, ak, bk, st); break;
     case NEOGEMM_VARIANT_T256x256_W4: e = launch_tile<256, 256, 2, 2>(a, ak, bk, st); break;
     case NEOGEMM_VARIANT_T128x128_W4: e = launch_tile<128, 128, 2, 2>(a, ak, bk, st); break;
-    case NEOGEMM_VARIANT_T256x128_W8: e = launch_tile<256, 128, 4, 2>(a, ak, bk, st); break;
-    case NEOGEMM_VARIANT_T128x256_W8: e = launch_tile<128, 256, 2, 4>(a, ak, bk, st); break;
+    case NEOGEMM_VARIANT_T256x128_W4: e = launch_tile<256, 128, 2, 2>(a, ak, bk, st); break;
+    case NEOGEMM_VARIANT_T128x256_W4: e = launch_tile<128, 256, 2, 2>(a, ak, bk, st); break;
     case NEOGEMM_VARIANT_T64x128_W4: e = launch_tile<64, 128, 1, 4>(a, ak, bk, st); break;
     case NEOGEMM_VARIANT_T128x128_W4S: e = launch_tile<128, 128, 1, 4>(a, ak, bk, st); break;
     case NEOGEMM_VARIANT_T192x256_W4: e = launch_tile<192, 256, 2, 2>(a, ak, bk, st); break;

@@ -46,8 +46,8 @@ extern "C" {
 #define NEOGEMM_VARIANT_T256x256_W8 2 /* 256x256, 8 wave64 (2x4) */
 #define NEOGEMM_VARIANT_T256x256_W4 3 /* 256x256, 4 wave64 (2x2): the default for large shapes */
 #define NEOGEMM_VARIANT_T128x128_W4 4 /* 128x128, 4 wave64 (2x2) */
-#define NEOGEMM_VARIANT_T256x128_W8 5 /* 256x128, 8 wave64 (4x2) */
-#define NEOGEMM_VARIANT_T128x256_W8 6 /* 128x256, 8 wave64 (2x4) */
+#define NEOGEMM_VARIANT_T256x128_W4 5 /* 256x128, 4 wave64 (2x2) */
+#define NEOGEMM_VARIANT_T128x256_W4 6 /* 128x256, 4 wave64 (2x2) */
 #define NEOGEMM_VARIANT_T64x128_W4 7  /* 64x128, 4 wave64 (1x4) */
 #define NEOGEMM_VARIANT_T128x128_W4S 8 /* 128x128, 4 wave64 (1x4) */
 /* Skinny M (or, with B [N,K], skinny N): a strip of 64 columns and all of K per workgroup, no split-K (decode shapes). */

@@ -21,8 +21,8 @@ from oracle import gemm_oracle as o
 
 pytestmark = pytest.mark.gpu
 
-TILE_VARIANTS = [g.VARIANT_T256x256_W8, g.VARIANT_T256x256_W4, g.VARIANT_T128x128_W4, g.VARIANT_T256x128_W8,
-                 g.VARIANT_T128x256_W8, g.VARIANT_T64x128_W4, g.VARIANT_T128x128_W4S, g.VARIANT_T192x256_W4]
+TILE_VARIANTS = [g.VARIANT_T256x256_W8, g.VARIANT_T256x256_W4, g.VARIANT_T128x128_W4, g.VARIANT_T256x128_W4,
+                 g.VARIANT_T128x256_W4, g.VARIANT_T64x128_W4, g.VARIANT_T128x128_W4S, g.VARIANT_T192x256_W4]
 ALL_VARIANTS = [g.VARIANT_GENERIC] + TILE_VARIANTS
 
 
