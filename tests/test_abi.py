@@ -62,6 +62,15 @@ def test_plan_for_the_benchmark_configs():
         s = max(s, _abi.plan(M, N, K, c_layout=1)[1])     # one query covers both output layouts
         assert _abi.workspace_bytes(M, N, K) == (s * M * N * 4 if s > 1 else 0)
     assert _abi.plan(1024, 1024, 32768)[1] > 1
+    # 3072^3 and 6144^3: 144 / 576 tiles of 256x256 fill 256 CUs badly, 192 / 768 tiles of 192x256 do better; the
+    # 192 rows must come from a K-major operand (A for a row-major C, B [N,K] for a column-major one)
+    for n in (3072, 6144):
+        assert _abi.plan(n, n, n) == (_abi.VARIANT_T192x256_W4, 1)
+        assert _abi.plan(n, n, n, b_layout=_abi.B_NK, c_layout=_abi.C_COL) == (_abi.VARIANT_T192x256_W4, 1)
+        assert _abi.plan(n, n, n, b_layout=_abi.B_KN, c_layout=_abi.C_COL)[0] != _abi.VARIANT_T192x256_W4
+    # tall shapes with a skinny N stream through the skinny kernel when B is [N,K]
+    assert _abi.plan(14336, 16, 4096, b_layout=_abi.B_NK) == (_abi.VARIANT_SKINNY16, 1)
+    assert _abi.plan(14336, 16, 4096, b_layout=_abi.B_KN)[0] not in (_abi.VARIANT_SKINNY16, _abi.VARIANT_GENERIC)
     # unaligned problems go to the generic kernel
     assert _abi.plan(100, 100, 100, aligned=False) == (_abi.VARIANT_GENERIC, 1)
     assert _abi.workspace_bytes(0, 5, 5) == 0 and _abi.workspace_bytes(5, 5, 0) == 0
