@@ -277,7 +277,13 @@ __device__ __forceinline__ bf16x8 with_half(bf16x8 f, i16x4 h, int which) {
 // PROF adds s_memtime stamps around the two waits of the main loop and writes, per wave,
 // {total, waiting for own loads, waiting at the barrier, epilogue} shader-clock cycles to p.prof — the
 // per-phase cycle buffer idea of the reference's harness (cublass/matmul.cu:99-106,149-165).
-template <int BM, int BN, int WGM, int WGN, bool AK, bool BK, bool PROF = false>
+// Images of B when both operands are K-major: three where the LDS has the room (one more tile of B in
+// flight: 64x128 tile -7 % at 1024^3, 128x256 -2.4 % at 8192^3), two for the 256x256 and 192x256 tiles, whose
+// A images and two of B fill the 160 KiB.  The 128x128 tile has both instances: three images make it 96 KiB,
+// one workgroup per CU, which pays when there is no second workgroup for the CU anyway (-10 % at 1536^3) and
+// costs when there is (+5..8 % at 4096^3 and 8192^3 with that tile).
+constexpr int b_images_both_kmajor(int bm, int bn) { return (bm + bn) * 384 <= 160 * 1024 ? 3 : 2; }
+template <int BM, int BN, int WGM, int WGN, bool AK, bool BK, bool PROF = false, int NB_KK = b_images_both_kmajor(BM, BN)>
 __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
   constexpr int NW = WGM * WGN;
   constexpr int WTM = BM / WGM, WTN = BN / WGN;
@@ -285,9 +291,9 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
   static_assert(WTM % 16 == 0 && WTN % 16 == 0, "wave tile must be a multiple of the 16x16 MFMA tile");
   static_assert(AK || BK, "at least one operand is K-major");
   // images per operand: four 32-deep slabs if MN-major; three 64-deep tiles if K-major, except that
-  // B gets by with two when both are K-major (160 KiB of LDS for a 256x256 tile either way)
+  // B gets by with NB_KK = two when both are K-major and the tile is large (160 KiB of LDS for a 256x256 tile either way)
   using OpA = Operand<BM, AK, NW, AK ? 3 : 4>;
-  using OpB = Operand<BN, BK, NW, BK ? (AK ? 2 : 3) : 4>;
+  using OpB = Operand<BN, BK, NW, BK ? (AK ? NB_KK : 3) : 4>;
   constexpr uint32_t A_BYTES = OpA::UNITS * OpA::IMG, LDS_BYTES = A_BYTES + OpB::UNITS * OpB::IMG;
   constexpr int IA = OpA::IPW, IB = OpB::IPW;  // this wave's loads per unit of A / of B
 
@@ -522,17 +528,19 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
   //     the sync before P2 needs Y slab 2t+3: all but Y slab 2t+4 and X tile t+3
   //   both K-major (A three images, B two): P0: B tile t+2, P1..P3: A tile t+3
   //     the sync before P0 needs A tile t+1 and B tile t+1: all but A tile t+2
+  //   (B three images: P0: B tile t+3; the sync before P0 keeps B tile t+2 and A tile t+2 in flight)
   //     no loads land between the sync before P0 and the reads of slab 2t+3: no second sync
-  constexpr int KEEP_ODD = (AK && BK) ? IA : (IA + IB + (AK ? IB : IA));
+  constexpr int KEEP_ODD = (AK && BK) ? IA + (NB_KK == 3 ? IB : 0) : (IA + IB + (AK ? IB : IA));
   constexpr int KEEP_EVEN = (AK && BK) ? -1 : IA + IB;
 
   // prologue: every image of both operands is requested, what slabs 0 and 1 need first, and only that
   // is waited for (units past K are requested too, fully masked: the counts below hold for any K).
   //   K-major A next to MN-major B: A0 B0 B1 | A1 B2 B3 A2      (mirrored if B is the K-major one)
-  //   both K-major:                 A0 B0 | A1 B1 A2
-  constexpr int KEEP_PRO = (AK && BK) ? 2 * IA + IB : 2 * IA + 2 * IB;
+  //   both K-major:                 A0 B0 | A1 B1 A2 (B2)
+  constexpr int KEEP_PRO = (AK && BK) ? 2 * IA + IB + (NB_KK == 3 ? IB : 0) : 2 * IA + 2 * IB;
   if constexpr (AK && BK) {
     burst_a(0); burst_b(0); burst_a(1); burst_b(1); burst_a(2);
+    if constexpr (NB_KK == 3) burst_b(2);
   } else if constexpr (AK) {
     burst_a(0); burst_b(0); burst_b(1); burst_a(1); burst_b(2); burst_b(3); burst_a(2);
   } else {
@@ -1046,7 +1054,8 @@ static const VariantInfo kVariants[NEOGEMM_VARIANT_COUNT] = {
 template <int BM, int BN, int WGM, int WGN>
 static hipError_t launch_tile(const TileArgs& a, bool ak, bool bk, hipStream_t st) {
   // A: three 64-deep images if K-major, else four 32-deep ones; B likewise, but two 64-deep ones if both are K-major
-  const size_t lds = (size_t)BM * (ak ? 384 : 256) + (size_t)BN * (bk && !ak ? 384 : 256);
+  // A: three 64-deep images if K-major, else four 32-deep ones; B likewise, but two or three 64-deep ones if both are K-major
+  size_t lds = (size_t)BM * (ak ? 384 : 256) + (size_t)BN * (bk ? (ak ? b_images_both_kmajor(BM, BN) * 128 : 384) : 256);
   dim3 grid(a.ntm * a.ntn, a.ksplit, a.batch), block(WGM * WGN * 64);
   auto go = [&](auto kern) -> hipError_t {
     static bool attr_done = false;  // per instantiation
@@ -1065,7 +1074,16 @@ static hipError_t launch_tile(const TileArgs& a, bool ak, bool bk, hipStream_t s
     }
     return hipErrorInvalidValue;
   }
-  if (ak && bk) return go(gemm_tile_kernel<BM, BN, WGM, WGN, true, true>);
+  if (ak && bk) {
+    if constexpr (BM == 128 && BN == 128) {
+      // more workgroups than CUs: two images of B, 80 KiB, so that two workgroups share a CU
+      if ((int64_t)a.ntm * a.ntn * a.ksplit * a.batch > 256) {
+        lds = (size_t)BM * 384 + (size_t)BN * 256;
+        return go(gemm_tile_kernel<BM, BN, WGM, WGN, true, true, false, 2>);
+      }
+    }
+    return go(gemm_tile_kernel<BM, BN, WGM, WGN, true, true>);
+  }
   if (ak && !bk) {
     if constexpr (BN >= 128 && (BN & (BN - 1)) == 0) return go(gemm_tile_kernel<BM, BN, WGM, WGN, true, false>);
   }
