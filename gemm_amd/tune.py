@@ -65,8 +65,8 @@ def tune_shape(M, N, K, nbuf=1, log=sys.stderr):
             if t < t_best:
                 best, t_best = (v, s), t
     t_model = min(t_model, time_us(lambda: call(None, 0)))   # the first measurement ran on a cold clock
-    if best == model:
-        t_best = t_model
+    if best == model or t_model <= t_best:
+        best, t_best = model, t_model
     print(f"{M}x{N}x{K}: model {model} {t_model:.2f} us, best {best} {t_best:.2f} us", file=log)
     return model, t_model, best, t_best
 
