@@ -1,19 +1,26 @@
 #!/usr/bin/env python3
 """Headline benchmark: BF16 GEMM M=N=K=8192 on one MI355X through the C ABI of libneogemm.so.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--all]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--preheat-ms T] [--all]
 
 Prints ONE JSON line.  A step is one GEMM (A [M,K] @ B [K,N], bf16 in, fp32 accumulate, bf16 out) on
-inputs already resident in HBM.  `value` is 2*M*N*K / (wall time per step) in TFLOP/s; `roofline` prices
-the kernel itself (HIP events on the launch stream) against the 2.5 PFLOP/s dense-BF16 peak;
-`cpu_baseline` is the oracle's fp32 torch.matmul timed on the host cores of the same box (a reported
-baseline, not a target); `vendor` is hipBLASLt/rocBLAS through torch.matmul on the same buffers.
+inputs already resident in HBM.  Order of events:
+  1. (before this process touches the GPU) the stand-alone harness gemm_amd/vendor_bench/matmul_bench runs as a
+     child: the matrix cores' power ceiling on N(0,1) operands (`roofline.power_ceiling`), and hipBLASLt (best of
+     its heuristic candidates) / rocBLAS / libneogemm on the same buffers, both layouts of B (`vendor`);
+  2. an untimed, time-based preheat of the very GEMM that is measured (`preheat_ms`): the chip is power-limited
+     on random data and the first launches after an idle period run slower until the clocks have settled;
+  3. W warm-up steps, then exactly K timed steps between two synchronisations: `value` = 2*M*N*K / wall time per
+     step.  The K steps are cut into batches, each bracketed by HIP events on the launch stream; the median batch
+     is `roofline.kernel_ms`, the list is `roofline.batch_ms`;
+  4. parity spot check against the CPU oracle, and the oracle's own fp32 product timed on the host cores
+     (`cpu_baseline`: a reported baseline, not a target).
 With --all the other benchmark configurations are timed too and reported under `other_configs`.
 """
 import argparse
 import json
-import math
 import os
+import subprocess
 import sys
 import time
 
@@ -22,22 +29,69 @@ sys.path.insert(0, ROOT)
 
 PEAK_TFLOPS = 2500.0   # MI355X dense BF16
 PEAK_HBM_GBS = 8000.0  # MI355X HBM3E
+MATMUL_BENCH = os.path.join(ROOT, "gemm_amd", "vendor_bench", "matmul_bench")
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "gemm_tile_256x256_w4_8192cubed_traffic.json")
 
 
-def time_gpu(fn, steps, warmup, torch):
-    """Wall time (host clock, sync on both sides) and HIP-event time per step."""
-    for _ in range(warmup):
-        fn()
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    e0.record()
-    for _ in range(steps):
-        fn()
-    e1.record()
-    torch.cuda.synchronize()
-    wall = (time.perf_counter() - t0) / steps
-    return wall * 1e3, e0.elapsed_time(e1) / steps
+def run_harness(args, env_extra=None, timeout=300):
+    """Run matmul_bench as a child and return its JSON lines (a list of dicts); [] if it is not built or fails."""
+    if not os.path.exists(MATMUL_BENCH):
+        return []
+    env = dict(os.environ)
+    env.update(env_extra or {})
+    try:
+        out = subprocess.run([MATMUL_BENCH] + [str(a) for a in args], env=env, capture_output=True, text=True,
+                             timeout=timeout).stdout
+    except (subprocess.TimeoutExpired, OSError):
+        return []
+    rows = []
+    for line in out.splitlines():
+        try:
+            rows.append(json.loads(line))
+        except ValueError:
+            pass
+    return rows
+
+
+def vendor_leg(M, N, K, preheat_ms):
+    """hipBLASLt best-of-heuristics, rocBLAS and libneogemm timed by one harness on the same buffers, B [K,N] and [N,K]."""
+    out = {"harness": "gemm_amd/vendor_bench/matmul_bench (child process, HIP events, median of 5 batches of 40, "
+                      f"{preheat_ms} ms preheat per library)"}
+    for bl, name in ((0, "b_kn"), (1, "b_nk")):
+        rows = run_harness([M, N, K, 40, bl], {"MATMUL_BENCH_PREHEAT_MS": str(preheat_ms)})
+        for r in rows:
+            if "lib" in r:
+                out[f"{r['lib']}_tflops_{name}"] = r["tflops"]
+                if r["lib"] == "hipblaslt":
+                    out[f"hipblaslt_algos_tried_{name}"] = r.get("algos_tried")
+            elif r.get("check") == "neogemm_vs_vendor":
+                out[f"rel_fro_vs_vendor_{name}"] = r["rel_fro"]
+    return out
+
+
+def power_ceiling(preheat_ms):
+    rows = [r for r in run_harness(["ceiling", preheat_ms]) if "ceiling" in r]
+    if not rows:
+        return None
+    out = {"what": "MFMA-only loop from registers, one wave per SIMD on 256 CUs, measured in this run before the GEMM "
+                   "(matmul_bench ceiling): the rate the chip's power limit allows the matrix cores alone",
+           "unit": "TFLOP/s"}
+    for r in rows:
+        short = "16x16x32" if "16x16x32" in r["ceiling"] else "32x32x16"
+        out[f"{short}_{r['operands']}"] = r["tflops"]
+        out[f"{short}_{r['operands']}_mhz"] = r["implied_mhz"]
+    return out
+
+
+def measured_traffic():
+    """HBM-side bytes per launch of the headline kernel from the tracked rocprofv3 --pmc summary (FETCH_SIZE and
+    WRITE_SIZE, each scaled by what the same counter reads for a plain copy of known size)."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            t = json.load(f)
+        return float(t["fetch_kib"]) * 1024.0 * float(t["fetch_scale"]) + float(t["write_kib"]) * 1024.0 * float(t["write_scale"])
+    except (OSError, ValueError, KeyError):
+        return None
 
 
 def main():
@@ -45,8 +99,11 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--preheat-ms", type=float, default=1500.0,
+                    help="untimed run of the measured GEMM before warm-up, until the clocks have settled")
     ap.add_argument("--all", action="store_true", help="also time the other benchmark configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline")
+    ap.add_argument("--no-vendor", action="store_true", help="skip the vendor-library and power-ceiling child runs")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy a few times, so that FETCH_SIZE / WRITE_SIZE "
                          "counters collected over this command can be scaled by what they read for a known size")
@@ -54,40 +111,86 @@ def main():
     if args.gpus != 1:
         sys.exit("bench.py: this build measures ONE GPU (the GEMM path has no multi-GPU part); run with --gpus 1. "
                  "A multi-GPU job would shard M or N with no exchange, so N GPUs run N copies of this kernel.")
+    M = N = K = 8192
+
+    # child runs first: this process has not initialised the GPU yet
+    ceiling = vendor = None
+    if not args.no_vendor:
+        ceiling = power_ceiling(1000)
+        vendor = vendor_leg(M, N, K, 1000)
 
     import torch
 
     import gemm_amd as g
+    from gemm_amd import _abi
     from oracle import gemm_oracle as o   # cpu_baseline leg and the parity spot-check only
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
-    M = N = K = 8192
     A, B = o.make_inputs(M, N, K, seed=0)          # N(0,1)/sqrt(K) bf16, generated on the CPU
     Ad, Bd = A.to(dev), B.to(dev)
     C = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
     variant, split_k = g.plan(M, N, K)
+    need = g.workspace_bytes(M, N, K)
+    ws = torch.empty(max(need, 16), dtype=torch.uint8, device=dev)
+    stream = torch.cuda.current_stream()
+    a_ptr, b_ptr, c_ptr, ws_ptr, st_ptr = Ad.data_ptr(), Bd.data_ptr(), C.data_ptr(), ws.data_ptr() if need else 0, stream.cuda_stream
 
     def step():
-        g.gemm_into(Ad, Bd, C, M, N, K, K, N, N, g.B_KN, g.C_ROW)
+        st = _abi.gemm_raw(a_ptr, b_ptr, c_ptr, M, N, K, K, N, N, g.B_KN, g.C_ROW, ws_ptr, need, st_ptr)
+        if st != _abi.OK:
+            raise g.NeoGemmError(st)
 
-    wall_ms, ev_ms = time_gpu(step, args.steps, args.warmup, torch)
+    # 2. preheat (time-based, untimed)
+    t_pre = time.perf_counter()
+    while (time.perf_counter() - t_pre) * 1e3 < args.preheat_ms:
+        for _ in range(20):
+            step()
+        torch.cuda.synchronize()
+    preheat_ms = (time.perf_counter() - t_pre) * 1e3
+    # 3. warm-up, then exactly --steps timed steps in event-bracketed batches
+    for _ in range(args.warmup):
+        step()
+    nb = min(10, args.steps) if args.steps >= 5 else args.steps
+    sizes = [args.steps // nb + (1 if i < args.steps % nb else 0) for i in range(nb)]
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(nb + 1)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ev[0].record(stream)
+    for i, n in enumerate(sizes):
+        for _ in range(n):
+            step()
+        ev[i + 1].record(stream)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    batch_ms = [ev[i].elapsed_time(ev[i + 1]) / sizes[i] for i in range(nb)]
+    kernel_ms = sorted(batch_ms)[nb // 2]
     flop = 2.0 * M * N * K
     value = flop / (wall_ms * 1e-3) / 1e12
-    achieved = flop / (ev_ms * 1e-3) / 1e12
+    achieved = flop / (kernel_ms * 1e-3) / 1e12
 
     # parity spot-check on a sample of rows (the full check lives in tests/test_gemm_gpu.py)
     idx = torch.randperm(M, generator=torch.Generator().manual_seed(1))[:128]
-    rep = o.parity_report(C[idx.to(dev)], A[idx], B)
+    got = C[idx.to(dev)].cpu()
+    ref = o.ref_gemm(A[idx], B)
+    rep = o.parity_report(got, A[idx], B, ref=ref)
     parity_ok = (rep["finite"] and rep["rel_fro"] <= o.TOL_REL_FRO and rep["max_ulp_floored"] <= o.TOL_ULP
-                 and rep["max_err_vs_bound"] <= 1.0)
+                 and rep["max_err_vs_bound"] <= 1.0 and rep["frac_gt1_ulp"] <= 2e-3)
+    ulp = o.ulp_distance(o.bits_of(got), o.bits_of(ref))
+    hist = {"0": int((ulp == 0).sum()), "1": int((ulp == 1).sum()), "2": int((ulp == 2).sum()),
+            "3-4": int(((ulp >= 3) & (ulp <= 4)).sum()), "5-16": int(((ulp >= 5) & (ulp <= 16)).sum()),
+            ">16": int((ulp > 16).sum())}
 
-    # vendor libraries on the same buffers (torch.matmul dispatches to hipBLASLt / rocBLAS)
-    vend_ms = time_gpu(lambda: torch.matmul(Ad, Bd, out=C), max(10, args.steps // 2), 5, torch)[1]
-    Bnk = Bd.t().contiguous()
-    vend_nt_ms = time_gpu(lambda: torch.matmul(Ad, Bnk.t(), out=C), max(10, args.steps // 2), 5, torch)[1]
-    ours_nt_ms = time_gpu(lambda: g.gemm_into(Ad, Bnk, C, M, N, K, K, K, N, g.B_NK, g.C_ROW), max(10, args.steps // 2), 5,
-                          torch)[1]
+    roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
+                "frac": round(achieved / PEAK_TFLOPS, 4),
+                # HBM-side bytes per launch from the tracked rocprofv3 --pmc summary; the algorithmic figure is 402.7e6
+                "traffic": measured_traffic(),
+                "kernel_ms": round(kernel_ms, 5), "batch_ms": [round(b, 5) for b in batch_ms],
+                "flop_per_launch": flop, "algorithmic_bytes": 2.0 * (M * K + K * N + M * N)}
+    if ceiling:
+        roofline["power_ceiling"] = ceiling
+        if ceiling.get("16x16x32_randn"):
+            roofline["frac_of_power_ceiling"] = round(achieved / ceiling["16x16x32_randn"], 4)
 
     out = {
         "metric": "BF16 GEMM TFLOP/s at 8192^3 on 1 MI355X; % of dense-BF16 peak",
@@ -96,6 +199,7 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "preheat_ms": round(preheat_ms, 1),
         "ms_per_step": round(wall_ms, 5),
         "higher_is_better": True,
         "scaling": "weak",
@@ -107,23 +211,41 @@ def main():
                    "b_layout": "[K,N]", "kernel_variant": g.VARIANT_NAMES[variant], "split_k": split_k,
                    "entry": "neogemm_bf16 (C ABI) on torch's current stream"},
         "pct_of_peak": round(100.0 * value / PEAK_TFLOPS, 2),
-        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved / PEAK_TFLOPS, 4),
-                     # HBM-side bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a plain copy
-                     # (profiles/gemm_tile_256x256_w4_8192cubed.txt); the algorithmic figure is 402.7e6
-                     "traffic": 1.762e9,
-                     "kernel_ms": round(ev_ms, 5), "flop_per_launch": flop},
-        "parity": {"ok": bool(parity_ok), "rows_checked": 128, **{k: rep[k] for k in ("max_ulp", "max_ulp_floored", "rel_fro")}},
-        "vendor": {"lib": "torch.matmul (hipBLASLt/rocBLAS)", "tflops_b_kn": round(flop / vend_ms / 1e9, 2),
-                   "tflops_b_nk": round(flop / vend_nt_ms / 1e9, 2), "neogemm_tflops_b_nk": round(flop / ours_nt_ms / 1e9, 2)},
+        "roofline": roofline,
+        "parity": {"ok": bool(parity_ok), "rows_checked": 128,
+                   **{k: rep[k] for k in ("max_ulp", "max_ulp_floored", "rel_fro", "frac_gt1_ulp", "max_err_vs_bound")},
+                   "raw_ulp_histogram": hist},
     }
+    if vendor:
+        out["vendor"] = vendor
+
+    def time_events(fn, steps, warmup):
+        for _ in range(warmup):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record(stream)
+        for _ in range(steps):
+            fn()
+        e1.record(stream)
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / steps
+
+    # torch.matmul (whatever torch dispatches to) on the same buffers, same process, clocks still warm
+    n_t = max(10, args.steps // 2)
+    Bnk = Bd.t().contiguous()
+    out["torch_matmul"] = {
+        "tflops_b_kn": round(flop / time_events(lambda: torch.matmul(Ad, Bd, out=C), n_t, 10) / 1e9, 2),
+        "tflops_b_nk": round(flop / time_events(lambda: torch.matmul(Ad, Bnk.t(), out=C), n_t, 10) / 1e9, 2),
+        "neogemm_tflops_b_nk": round(flop / time_events(
+            lambda: g.gemm_into(Ad, Bnk, C, M, N, K, K, K, N, g.B_NK, g.C_ROW), n_t, 10) / 1e9, 2)}
 
     if args.all:
         others = []
         for (m, n, k) in ((512, 512, 512), (4096, 4096, 4096), (16, 14336, 4096), (64, 14336, 4096),
                           (128, 14336, 4096), (3000, 5120, 3584), (1024, 1024, 32768)):
             a, b = o.make_inputs(m, n, k, seed=1)
-            nbuf = 6 if m <= 128 else 1   # rotate weights larger than the 256 MB last-level cache
+            nbuf = 8 if m <= 128 else 1   # rotate weights larger than the 256 MB last-level cache
             ad, bds = a.to(dev), [b.to(dev).clone() for _ in range(nbuf)]
             c = torch.empty(m, n, dtype=torch.bfloat16, device=dev)
             it = [0]
@@ -136,14 +258,14 @@ def main():
                 torch.matmul(ad, bds[it[0] % nbuf], out=c)
                 it[0] += 1
 
-            ms = time_gpu(f, 200 if m * n * k < 2e11 else 50, 20, torch)[1]
-            vms = time_gpu(fv, 200 if m * n * k < 2e11 else 50, 20, torch)[1]
+            ms = time_events(f, 200 if m * n * k < 2e11 else 50, 20)
+            vms = time_events(fv, 200 if m * n * k < 2e11 else 50, 20)
             fl, by = 2.0 * m * n * k, 2.0 * (m * k + k * n + m * n)
             v, s = g.plan(m, n, k)
             others.append({"M": m, "N": n, "K": k, "ms": round(ms, 5), "tflops": round(fl / ms / 1e9, 2),
                            "pct_of_2500": round(fl / ms / 1e9 / 25.0, 2), "gbps": round(by / ms / 1e6, 1),
                            "pct_of_8000": round(by / ms / 1e6 / 80.0, 2), "variant": g.VARIANT_NAMES[v], "split_k": s,
-                           "vendor_ms": round(vms, 5)})
+                           "torch_matmul_ms": round(vms, 5)})
         out["other_configs"] = others
 
     if args.calibrate_copy:
@@ -155,17 +277,17 @@ def main():
         out["calibration_copy_bytes"] = 256 << 20
 
     if not args.no_cpu:
-        # host baseline: the oracle's fp32 product, one full-size GEMM after a small warm-up
+        # host baseline: the oracle's fp32 product, full-size GEMMs after a small warm-up
         nthreads = torch.get_num_threads()
         o.ref_gemm_f32(A[:256], B)
         times = []
-        for _ in range(3):
+        for _ in range(5):
             t0 = time.perf_counter()
             o.ref_gemm_f32(A, B)
             times.append(time.perf_counter() - t0)
-        dt = sorted(times)[1]
+        dt = sorted(times)[len(times) // 2]
         out["cpu_baseline"] = {"value": round(flop / dt / 1e12, 4), "unit": "TFLOP/s", "cores": nthreads, "kind": "port",
-                               "sample": f"full M=N=K=8192 fp32 torch.matmul on the host, median of 3 ({dt:.1f} s each), "
+                               "sample": f"full M=N=K=8192 fp32 torch.matmul on the host, median of 5 ({dt:.1f} s each), "
                                          f"{os.cpu_count()} logical CPUs visible",
                                "seconds": round(dt, 2)}
     print(json.dumps(out), flush=True)

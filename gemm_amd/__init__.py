@@ -33,10 +33,18 @@ def _check(t, name):
 
 
 def _workspace(device, nbytes):
-    ws = _workspaces.get(device)
-    if ws is None or ws.numel() < nbytes:
-        ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
-        _workspaces[device] = ws
+    """Split-K scratch for torch's current stream on `device`: one buffer per (device, stream), so that GEMMs on
+    different streams never share partials.  A buffer is allocated while its stream is current and used on that
+    stream only, so when a larger one replaces it the caching allocator reuses the block in that stream's order."""
+    with torch.cuda.device(device):
+        key = (device.index if device.index is not None else torch.cuda.current_device(),
+               torch.cuda.current_stream().cuda_stream)
+        ws = _workspaces.get(key)
+        if ws is None or ws.numel() < nbytes:
+            _workspaces.pop(key, None)
+            ws = None
+            ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+            _workspaces[key] = ws
     return ws
 
 

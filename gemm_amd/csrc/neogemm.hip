@@ -4,14 +4,16 @@
 // the fp32-accumulated dot product of a row of A with a row/column of B, rounded once to bf16 with
 // round-to-nearest-even.  How it is computed shares nothing with it: the reference stages 64x64 tiles
 // with TMA and issues WGMMA from one warpgroup (v01.cu:215-237); here a workgroup of wave64s owns a
-// 256x256 (or smaller) macro-tile, stages 64-deep K slabs with direct-to-LDS buffer loads into a
-// double-buffered, XOR-swizzled LDS image, and feeds v_mfma_f32_16x16x32_bf16 from ds_read_b128 /
-// ds_read_b64_tr_b16.
+// 256x256 (or smaller) macro-tile, stages K with direct-to-LDS buffer loads into a ring of three or four
+// XOR-swizzled LDS images per operand (64-deep tiles of a K-major operand, 32-deep slabs of an MN-major
+// one), and feeds v_mfma_f32_16x16x32_bf16 from ds_read_b128 / ds_read_b64_tr_b16.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stdio.h>
 #include <stdlib.h>
 
+#include <atomic>
+#include <mutex>
 #include <type_traits>
 #include <string>
 #include <utility>
@@ -47,7 +49,8 @@ static constexpr uint32_t VOFF_BIAS = 3 * 1024;
 //   logical chunk c of row r lives at physical chunk c ^ swz_k(r).  64 deep, not 32, so that one
 //   direct-to-LDS instruction (8 rows x 128 B) asks the L2 for whole 128-byte lines: with 64-byte
 //   pieces the vector L1 issues twice the requests and the wave that issues the load is held up
-//   roughly in proportion to the number of requests.  Two images per operand (double buffer).
+//   roughly in proportion to the number of requests.  Three images per operand (two for B of the largest
+//   tiles when both operands are K-major).
 // MN-major operand (the K index is the slow one: B[K,N]) — image of a 32-deep SLAB:
 //   32 x (ROWS*2) B, k-row at k*ROWS*2; logical chunk c (8 columns) of k-row k lives at physical
 //   chunk c ^ swz_mn(k).  Rows are whole lines already.  Read back with ds_read_b64_tr_b16: in each
@@ -642,8 +645,9 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
   if (stage) {
     if constexpr (CAN_STAGE) {
       // every wave is done with the slab images (its LDS reads have returned: the MFMAs that used them
-      // were issued; wait anyway) before any wave overwrites them
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      // were issued; wait anyway) before any wave overwrites them; so are its direct-to-LDS loads (when K is
+      // short the prologue's fully masked zero fills of later images may still be in flight)
+      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
       __builtin_amdgcn_s_barrier();
       asm volatile("" ::: "memory");
       const uint32_t region = lds0 + (uint32_t)wave * (WTM * WTN * 2);
@@ -1014,14 +1018,16 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
 __global__ __launch_bounds__(256) void gemm_generic_kernel(const __bf16* __restrict__ A, const __bf16* __restrict__ B,
                                                            __bf16* C, int M, int N, int K, long sam, long sak,
                                                            long sbk, long sbn, long scm, long scn, float alpha,
-                                                           float beta, long bsa, long bsb, long bsc) {
+                                                           float beta, long bsa, long bsb, long bsc, unsigned nbx) {
   A += (size_t)blockIdx.z * bsa;  // problem blockIdx.z of the batch
   B += (size_t)blockIdx.z * bsb;
   C += (size_t)blockIdx.z * bsc;
   __shared__ float sa[16][17];
   __shared__ float sb[16][17];
   const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
-  const long row = (long)blockIdx.y * 16 + ty, col = (long)blockIdx.x * 16 + tx;
+  // blockIdx.x counts 16x16 output blocks row by row (nbx per block row): grid.y is limited to 65535
+  const unsigned by = blockIdx.x / nbx, bx = blockIdx.x - by * nbx;
+  const long row = (long)by * 16 + ty, col = (long)bx * 16 + tx;
   float acc = 0.f;
   for (int k0 = 0; k0 < K; k0 += 16) {
     // sa[ty][tx] = A(row, k0+tx); sb[ty][tx] = B(k0+ty, col)
@@ -1051,19 +1057,30 @@ static const VariantInfo kVariants[NEOGEMM_VARIANT_COUNT] = {
     {16, 64, 4}, {32, 64, 4}, {64, 64, 4}, {192, 256, 4},
 };
 
+// Raise a kernel's dynamic-LDS limit once per (instantiation, device): the attribute belongs to the current
+// device's copy of the function.  `done` holds one bit per device index.
+template <class Kern>
+static hipError_t allow_lds(Kern kern, size_t lds, std::atomic<uint64_t>& done) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  const uint64_t bit = 1ull << (dev & 63);
+  if (dev > 63 || !(done.load(std::memory_order_acquire) & bit)) {
+    e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return e;
+    done.fetch_or(bit, std::memory_order_release);
+  }
+  return hipSuccess;
+}
+
 template <int BM, int BN, int WGM, int WGN>
 static hipError_t launch_tile(const TileArgs& a, bool ak, bool bk, hipStream_t st) {
-  // A: three 64-deep images if K-major, else four 32-deep ones; B likewise, but two 64-deep ones if both are K-major
   // A: three 64-deep images if K-major, else four 32-deep ones; B likewise, but two or three 64-deep ones if both are K-major
   size_t lds = (size_t)BM * (ak ? 384 : 256) + (size_t)BN * (bk ? (ak ? b_images_both_kmajor(BM, BN) * 128 : 384) : 256);
   dim3 grid(a.ntm * a.ntn, a.ksplit, a.batch), block(WGM * WGN * 64);
   auto go = [&](auto kern) -> hipError_t {
-    static bool attr_done = false;  // per instantiation
-    if (!attr_done) {
-      hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-      if (e != hipSuccess) return e;
-      attr_done = true;
-    }
+    static std::atomic<uint64_t> attr_done{0};  // per instantiation
+    if (hipError_t e = allow_lds(kern, lds, attr_done); e != hipSuccess) return e;
     kern<<<grid, block, lds, st>>>(a);
     return hipGetLastError();
   };
@@ -1191,13 +1208,14 @@ static void plan_model(int64_t M, int64_t N, int64_t K, bool aligned, int c_layo
 }
 
 // Tuned choices override the model: the file named by the environment variable NEOGEMM_PLAN_TABLE, read
-// once, holds a JSON array of objects {"M":..,"N":..,"K":..,"c_layout":..,"variant":..,"split_k":..}
-// (what gemm_amd/tune.py writes; c_layout defaults to 0).  The reference fixes tile and stage counts at
+// once, holds a JSON array of objects {"M":..,"N":..,"K":..,"b_layout":..,"c_layout":..,"variant":..,"split_k":..}
+// (what gemm_amd/tune.py writes; b_layout and c_layout default to 0); an entry applies to calls with exactly
+// its shape and layouts, since the kernels behind the layouts differ.  The reference fixes tile and stage counts at
 // compile time (v01.cu:275-278); this is the run-time counterpart.  Entries with an unknown variant or a
 // split below 1 are ignored, and so is an unreadable file.
 struct PlanEntry {
   int64_t M, N, K;
-  int c_layout, variant, split_k;
+  int b_layout, c_layout, variant, split_k;
 };
 static const std::vector<PlanEntry>& plan_table() {
   static const std::vector<PlanEntry> table = [] {
@@ -1224,10 +1242,11 @@ static const std::vector<PlanEntry>& plan_table() {
         if (at == std::string::npos) return dflt;
         return strtoll(obj.c_str() + at + 1, nullptr, 10);
       };
-      PlanEntry e{field("M", -1), field("N", -1), field("K", -1), (int)field("c_layout", 0), (int)field("variant", -1),
-                  (int)field("split_k", 0)};
+      PlanEntry e{field("M", -1), field("N", -1), field("K", -1), (int)field("b_layout", 0), (int)field("c_layout", 0),
+                  (int)field("variant", -1), (int)field("split_k", 0)};
       if (e.M > 0 && e.N > 0 && e.K > 0 && e.variant > NEOGEMM_VARIANT_AUTO && e.variant < NEOGEMM_VARIANT_COUNT &&
-          e.split_k >= 1 && e.split_k <= 64 && (e.c_layout == NEOGEMM_C_ROW || e.c_layout == NEOGEMM_C_COL))
+          e.split_k >= 1 && e.split_k <= 64 && (e.c_layout == NEOGEMM_C_ROW || e.c_layout == NEOGEMM_C_COL) &&
+          (e.b_layout == NEOGEMM_B_KN || e.b_layout == NEOGEMM_B_NK))
         t.push_back(e);
       pos = end + 1;
     }
@@ -1239,13 +1258,27 @@ static void plan(int64_t M, int64_t N, int64_t K, bool aligned, int c_layout, in
                  int64_t batch = 1, int b_layout = NEOGEMM_B_KN) {
   if (aligned && K > 0 && batch == 1) {
     for (const PlanEntry& e : plan_table())
-      if (e.M == M && e.N == N && e.K == K && e.c_layout == c_layout) {
+      if (e.M == M && e.N == N && e.K == K && e.c_layout == c_layout && e.b_layout == b_layout) {
         *variant = e.variant;
         *split_k = e.variant == NEOGEMM_VARIANT_GENERIC ? 1 : e.split_k;
         return;
       }
   }
   plan_model(M, N, K, aligned, c_layout, variant, split_k, batch, b_layout);
+}
+
+// The largest split-K factor plan() returns for this shape over the four (b_layout, c_layout) combinations a call can
+// name (the kernels, and so the plans, differ between them): the workspace queries bound every call for the shape,
+// the reference's own (B [N,K], column-major C: nemgemmV03.cu:346, v01.cu:246,252) included.
+static int max_planned_split(int64_t M, int64_t N, int64_t K, int64_t batch) {
+  int best = 1;
+  for (int bl : {NEOGEMM_B_KN, NEOGEMM_B_NK})
+    for (int cl : {NEOGEMM_C_ROW, NEOGEMM_C_COL}) {
+      int v, s;
+      plan(M, N, K, true, cl, &v, &s, batch, bl);
+      if (s > best) best = s;
+    }
+  return best;
 }
 
 // A batch of `count` problems of one shape; strides in elements between consecutive problems (0: shared operand).
@@ -1289,10 +1322,12 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
   if (v == NEOGEMM_VARIANT_GENERIC) {
     const long sbk = b_layout == NEOGEMM_B_KN ? ldb : 1, sbn = b_layout == NEOGEMM_B_KN ? 1 : ldb;
     const long scm = c_layout == NEOGEMM_C_ROW ? ldc : 1, scn = c_layout == NEOGEMM_C_ROW ? 1 : ldc;
-    dim3 grid(ceil_div(N, 16), ceil_div(M, 16), (unsigned)bt.count);
-    if (grid.y > 65535u) return NEOGEMM_ERR_UNSUPPORTED;
+    const int64_t nbx = ceil_div(N, 16), nblocks = nbx * ceil_div(M, 16);
+    if (nblocks > 0x7fffffff) return NEOGEMM_ERR_UNSUPPORTED;
+    dim3 grid((unsigned)nblocks, 1, (unsigned)bt.count);
     gemm_generic_kernel<<<grid, 256, 0, st>>>((const __bf16*)A, (const __bf16*)B, (__bf16*)C, (int)M, (int)N, (int)K,
-                                              lda, 1, sbk, sbn, scm, scn, alpha, beta, bt.sa, bt.sb, bt.sc);
+                                              lda, 1, sbk, sbn, scm, scn, alpha, beta, bt.sa, bt.sb, bt.sc,
+                                              (unsigned)nbx);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
       fprintf(stderr, "neogemm: generic kernel launch failed: %s\n", hipGetErrorString(e));
@@ -1328,12 +1363,8 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
       ccol = !ccol;  // a row-major C[m][n] is the column-major C^T
     }
     auto go = [&](auto kern, size_t lds) -> hipError_t {
-      static bool attr_done = false;  // per instantiation
-      if (!attr_done) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return e;
-        attr_done = true;
-      }
+      static std::atomic<uint64_t> attr_done{0};  // per instantiation
+      if (hipError_t e = allow_lds(kern, lds, attr_done); e != hipSuccess) return e;
       kern<<<dim3(ceil_div(sa.N, 64)), 256, lds, st>>>(sa);
       return hipGetLastError();
     };
@@ -1471,10 +1502,7 @@ int neogemm_bf16_batched(const void* A, const void* B, void* C, int64_t M, int64
 
 size_t neogemm_bf16_batched_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t batch) {
   if (M <= 0 || N <= 0 || K <= 0 || batch <= 0) return 0;
-  int v, s, v2, s2;
-  neogemm::plan(M, N, K, true, NEOGEMM_C_ROW, &v, &s, batch);
-  neogemm::plan(M, N, K, true, NEOGEMM_C_COL, &v2, &s2, batch);
-  if (s2 > s) s = s2;
+  const int s = neogemm::max_planned_split(M, N, K, batch);
   return s > 1 ? (size_t)s * (size_t)M * (size_t)N * sizeof(float) * (size_t)batch : 0;
 }
 
@@ -1503,12 +1531,7 @@ size_t neogemm_bf16_profile_bytes(int64_t M, int64_t N, int variant) {
 
 size_t neogemm_bf16_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   if (M <= 0 || N <= 0 || K <= 0) return 0;
-  int v, s;
-  // the larger of the two output layouts' needs, so that one query covers any call for this shape
-  int v2, s2;
-  neogemm::plan(M, N, K, true, NEOGEMM_C_ROW, &v, &s);
-  neogemm::plan(M, N, K, true, NEOGEMM_C_COL, &v2, &s2);
-  if (s2 > s) s = s2;
+  const int s = neogemm::max_planned_split(M, N, K, 1);
   return s > 1 ? (size_t)s * (size_t)M * (size_t)N * sizeof(float) : 0;
 }
 

@@ -10,14 +10,15 @@
 //  * arguments are validated (the reference only checks dtype through data_ptr<>, nemgemmV03.cu:349-351)
 //    and failures raise instead of printing to stderr (nemgemmV03.cu:387-390);
 //  * the launch goes to torch's current stream, not the legacy default stream (nemgemmV03.cu:383);
-//  * no state is cached between calls (the reference caches TMA descriptors keyed on shape only,
-//    nemgemmV03.cu:27-30,359-371, which goes stale when another tensor of the same shape is passed).
+//  * no state tied to a tensor is cached between calls (the reference caches TMA descriptors keyed on shape
+//    only, nemgemmV03.cu:27-30,359-371, which goes stale when another tensor of the same shape is passed); the
+//    only state kept is a split-K scratch buffer per (device, stream).
 #include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 #include <torch/extension.h>
 
+#include <map>
 #include <string>
-#include <vector>
 
 #include "neogemm.h"
 
@@ -34,17 +35,24 @@ void check_operand(const torch::Tensor& t, const char* name) {
 bool row_major(const torch::Tensor& t) { return t.size(1) <= 1 || t.stride(1) == 1; }
 int64_t row_ld(const torch::Tensor& t) { return t.size(0) <= 1 ? std::max<int64_t>(t.size(1), 1) : t.stride(0); }
 
-// Per-device split-K scratch.  Grown on demand through torch's caching allocator and kept; launches
-// on one stream are ordered, and a tensor replaced here stays alive until the stream that used it has
-// passed (the caching allocator defers reuse of blocks recorded on a stream).
-torch::Tensor& workspace_for(const torch::Tensor& like, size_t bytes) {
-  static thread_local std::vector<torch::Tensor> ws(64);
-  const int dev = like.get_device();
-  TORCH_CHECK(dev >= 0 && dev < 64, "unexpected device index ", dev);
-  if (!ws[dev].defined() || (size_t)ws[dev].numel() < bytes) {
-    ws[dev] = torch::empty({(int64_t)bytes}, like.options().dtype(torch::kUInt8));
+// Split-K scratch, one buffer per (device, stream): two GEMMs on two streams of one device must not share their
+// partials, and a buffer is only ever used on the stream that was current when the caching allocator handed it out,
+// which is the stream whose order the allocator follows when the block is reused.  So dropping a buffer that has
+// become too small is safe: its block goes back to that stream's pool and is handed out again only to work queued
+// on that same stream, behind the kernels that still use it.  The cache is per host thread.
+struct WorkspaceKey {
+  int device;
+  hipStream_t stream;
+  bool operator<(const WorkspaceKey& o) const { return device != o.device ? device < o.device : stream < o.stream; }
+};
+torch::Tensor& workspace_for(const torch::Tensor& like, hipStream_t stream, size_t bytes) {
+  static thread_local std::map<WorkspaceKey, torch::Tensor> ws;
+  torch::Tensor& t = ws[WorkspaceKey{(int)like.get_device(), stream}];
+  if (!t.defined() || (size_t)t.numel() < bytes) {
+    t = torch::Tensor();  // give the old block back first
+    t = torch::empty({(int64_t)bytes}, like.options().dtype(torch::kUInt8));
   }
-  return ws[dev];
+  return t;
 }
 
 void run(const torch::Tensor& A, const torch::Tensor& B, torch::Tensor& C, int64_t M, int64_t N, int64_t K,
@@ -52,9 +60,9 @@ void run(const torch::Tensor& A, const torch::Tensor& B, torch::Tensor& C, int64
   // PyTorch-ROCm names its HIP devices "cuda"; these are the guard and stream accessors for that naming
   c10::hip::HIPGuardMasqueradingAsCUDA guard(A.device());
   const size_t need = neogemm_bf16_workspace_bytes(M, N, K);
-  void* ws = nullptr;
-  if (need) ws = workspace_for(A, need).data_ptr();
   hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(A.get_device()).stream();
+  void* ws = nullptr;
+  if (need) ws = workspace_for(A, stream, need).data_ptr();
   const int st = (alpha == 1.f && beta == 0.f)
                      ? neogemm_bf16(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, lda, ldb, ldc, b_layout,
                                     c_layout, ws, need, (void*)stream)
@@ -130,9 +138,9 @@ torch::Tensor bmm(torch::Tensor A, torch::Tensor B) {
   if (batch == 0 || M == 0 || N == 0) return C;
   c10::hip::HIPGuardMasqueradingAsCUDA guard(A.device());
   const size_t need = neogemm_bf16_batched_workspace_bytes(M, N, K, batch);
-  void* ws = nullptr;
-  if (need) ws = workspace_for(A, need).data_ptr();
   hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(A.get_device()).stream();
+  void* ws = nullptr;
+  if (need) ws = workspace_for(A, stream, need).data_ptr();
   const int st = neogemm_bf16_batched(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, std::max<int64_t>(K, 1),
                                       std::max<int64_t>(N, 1), std::max<int64_t>(N, 1), M * K, B.dim() == 3 ? K * N : 0,
                                       M * N, batch, NEOGEMM_B_KN, NEOGEMM_C_ROW, ws, need, (void*)stream);

@@ -4,7 +4,9 @@
     NEOGEMM_PLAN_TABLE=plan_table.json python bench.py        # the library reads the table once, at first use
 
 The table is the JSON array libneogemm.so looks up before its cost model (neogemm_bf16_plan): objects
-{"M","N","K","c_layout","variant","split_k"}.  Only shapes whose best measured candidate beats the model's
+{"M","N","K","b_layout","c_layout","variant","split_k"}; an entry applies to exactly its shape and layouts
+(--b-layout 1 tunes B [N,K], --c-layout 1 a column-major C: --b-layout 1 --c-layout 1 is the reference's call,
+nemgemmV03.cu:343-391).  Only shapes whose best measured candidate beats the model's
 choice by more than --margin are written.  The reference has nothing of the kind: its tile and stage
 counts are template arguments (v01.cu:275-278, 304-311).
 """
@@ -16,7 +18,7 @@ import sys
 import torch
 
 from . import _abi, gemm_into, plan
-from ._abi import B_KN, C_ROW, ERR_UNSUPPORTED, NeoGemmError
+from ._abi import B_KN, B_NK, C_COL, C_ROW, ERR_UNSUPPORTED, NeoGemmError
 
 CANDIDATE_VARIANTS = (_abi.VARIANT_T256x256_W4, _abi.VARIANT_T256x256_W8, _abi.VARIANT_T128x256_W4,
                       _abi.VARIANT_T256x128_W4, _abi.VARIANT_T128x128_W4, _abi.VARIANT_T64x128_W4,
@@ -37,19 +39,20 @@ def time_us(fn, warmup=5, iters=30):
     return start.elapsed_time(stop) * 1000.0 / iters
 
 
-def tune_shape(M, N, K, nbuf=1, log=sys.stderr):
-    """Returns (model choice, its time, best choice, its time) for row-major A [M,K], B [K,N], C [M,N]."""
+def tune_shape(M, N, K, nbuf=1, log=sys.stderr, b_layout=B_KN, c_layout=C_ROW):
+    """Returns (model choice, its time, best choice, its time) for A [M,K], B in `b_layout`, C in `c_layout`."""
     gen = torch.Generator().manual_seed(0)
     A = (torch.randn(M, K, generator=gen) / math.sqrt(K)).to(torch.bfloat16).cuda()
-    Bs = [(torch.randn(K, N, generator=gen) / math.sqrt(K)).to(torch.bfloat16).cuda() for _ in range(nbuf)]
-    C = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+    b_shape = (K, N) if b_layout == B_KN else (N, K)
+    Bs = [(torch.randn(*b_shape, generator=gen) / math.sqrt(K)).to(torch.bfloat16).cuda() for _ in range(nbuf)]
+    C = torch.empty((M, N) if c_layout == C_ROW else (N, M), dtype=torch.bfloat16, device="cuda")
     turn = [0]
 
     def call(variant, split):
         turn[0] += 1
-        gemm_into(A, Bs[turn[0] % nbuf], C, M, N, K, K, N, N, B_KN, C_ROW, variant, split, 0)
+        gemm_into(A, Bs[turn[0] % nbuf], C, M, N, K, K, b_shape[1], C.shape[1], b_layout, c_layout, variant, split, 0)
 
-    model = plan(M, N, K)
+    model = plan(M, N, K, b_layout, c_layout)
     t_model = time_us(lambda: call(None, 0))
     best, t_best = model, t_model
     for v in CANDIDATE_VARIANTS:
@@ -67,7 +70,7 @@ def tune_shape(M, N, K, nbuf=1, log=sys.stderr):
     t_model = min(t_model, time_us(lambda: call(None, 0)))   # the first measurement ran on a cold clock
     if best == model or t_model <= t_best:
         best, t_best = model, t_model
-    print(f"{M}x{N}x{K}: model {model} {t_model:.2f} us, best {best} {t_best:.2f} us", file=log)
+    print(f"{M}x{N}x{K} b{b_layout} c{c_layout}: model {model} {t_model:.2f} us, best {best} {t_best:.2f} us", file=log)
     return model, t_model, best, t_best
 
 
@@ -77,15 +80,18 @@ def main():
     ap.add_argument("--out", required=True)
     ap.add_argument("--margin", type=float, default=0.03, help="minimum relative gain over the model's choice")
     ap.add_argument("--nbuf", type=int, default=1, help="rotate this many B buffers (streaming shapes)")
+    ap.add_argument("--b-layout", type=int, default=B_KN, choices=(B_KN, B_NK), help="0: B [K,N], 1: B [N,K]")
+    ap.add_argument("--c-layout", type=int, default=C_ROW, choices=(C_ROW, C_COL), help="0: row-major C, 1: column-major")
     args = ap.parse_args()
     if not torch.cuda.is_available():
         sys.exit("tuning needs a GPU")
     table = []
     for sh in args.shapes:
         M, N, K = (int(x) for x in sh.lower().split("x"))
-        model, t_model, best, t_best = tune_shape(M, N, K, args.nbuf)
+        model, t_model, best, t_best = tune_shape(M, N, K, args.nbuf, b_layout=args.b_layout, c_layout=args.c_layout)
         if best != model and t_best < t_model * (1.0 - args.margin):
-            table.append({"M": M, "N": N, "K": K, "c_layout": C_ROW, "variant": best[0], "split_k": best[1]})
+            table.append({"M": M, "N": N, "K": K, "b_layout": args.b_layout, "c_layout": args.c_layout,
+                          "variant": best[0], "split_k": best[1]})
     with open(args.out, "w") as f:
         json.dump(table, f, indent=1)
     print(f"{len(table)} entries written to {args.out}", file=sys.stderr)

@@ -8,8 +8,16 @@
 // last-level cache, and cross-checks the libraries against each other.
 //
 //   matmul_bench M N K [reps=100] [b_layout=0|1] [variant=0] [split_k=0] [group_m=0] [nbuf=1]
+//   matmul_bench ceiling [preheat_ms=1000]
 //
 // One line of JSON per library on stdout.
+//
+// `ceiling` measures what the matrix cores sustain with nothing else going on: every wave runs the MFMA
+// sequence of a 128x128 wave tile (the 256x256 GEMM tile's share of one wave) from registers, no memory
+// traffic at all, one wave per SIMD on all 256 CUs, with all-zero operands and with N(0,1)/sqrt(8192) bf16
+// operands (two register sets alternating, so that the operand buses toggle as they do on fresh data).  On
+// zeros the chip holds its top clock; on random data it is power-limited and the clock drops: that rate, not
+// the data-sheet peak, bounds any GEMM kernel on such inputs on this chip.
 #include <hip/hip_runtime.h>
 #include <hipblaslt/hipblaslt.h>
 #include <rocblas/rocblas.h>
@@ -55,6 +63,13 @@ static float bf2f(uint16_t h) {
   return f;
 }
 
+// MATMUL_BENCH_PREHEAT_MS (environment, default 0): before timing a library, run it for that long, so that the
+// chip's clocks have settled under that very load (the first launches after an idle period run slower).
+static double preheat_ms_from_env() {
+  const char* e = getenv("MATMUL_BENCH_PREHEAT_MS");
+  return e ? atof(e) : 0.0;
+}
+
 template <class F>
 static double time_ms(F&& launch, int reps, hipStream_t st) {
   hipEvent_t a, b;
@@ -63,6 +78,16 @@ static double time_ms(F&& launch, int reps, hipStream_t st) {
   const int warm = std::max(3, reps / 10);
   for (int i = 0; i < warm; ++i) launch(i);
   HIP_OK(hipStreamSynchronize(st));
+  static const double preheat = preheat_ms_from_env();
+  for (double heated = 0.0; heated < preheat;) {
+    HIP_OK(hipEventRecord(a, st));
+    for (int i = 0; i < warm; ++i) launch(i);
+    HIP_OK(hipEventRecord(b, st));
+    HIP_OK(hipEventSynchronize(b));
+    float t;
+    HIP_OK(hipEventElapsedTime(&t, a, b));
+    heated += t > 0.f ? t : 1.0;
+  }
   // median of 5 batches
   std::vector<double> ms;
   for (int batch = 0; batch < 5; ++batch) {
@@ -89,9 +114,139 @@ static void report(const char* lib, int64_t M, int64_t N, int64_t K, int bl, dou
   fflush(stdout);
 }
 
+// ---- MFMA-only power ceiling -------------------------------------------------------------------
+typedef __attribute__((ext_vector_type(8))) __bf16 cbf16x8;
+typedef __attribute__((ext_vector_type(4))) float cf32x4;
+typedef __attribute__((ext_vector_type(16))) float cf32x16;
+
+// frags: [set 2][operand 2][8][256 threads] bf16x8.  One pass = the MFMAs of a 128x128x32 wave-tile step:
+// 64 x v_mfma_f32_16x16x32_bf16 (8x8 tiles of 16x16), or 32 x v_mfma_f32_32x32x16_bf16 (4x4 tiles of 32x32, two
+// 16-deep steps).  Accumulators sit in the 256 AGPRs and are written in place, as in the GEMM kernel.
+template <bool BIG>
+__global__ __launch_bounds__(256) void mfma_ceiling_kernel(const cbf16x8* frags, float* out, int passes) {
+  cbf16x8 a[2][8], b[2][8];
+#pragma unroll
+  for (int s = 0; s < 2; ++s)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      a[s][i] = frags[((s * 2 + 0) * 8 + i) * 256 + threadIdx.x];
+      b[s][i] = frags[((s * 2 + 1) * 8 + i) * 256 + threadIdx.x];
+    }
+  float total = 0.f;
+  if constexpr (!BIG) {
+    cf32x4 acc[8][8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[i][j] = cf32x4{0.f, 0.f, 0.f, 0.f};
+    for (int p = 0; p < passes; p += 2) {
+#pragma unroll
+      for (int s = 0; s < 2; ++s)
+#pragma unroll
+        for (int c = 0; c < 8; ++c)
+#pragma unroll
+          for (int i = 0; i < 8; ++i)
+            asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[i][c]) : "v"(b[s][c]), "v"(a[s][i]));
+    }
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        asm volatile("" : "+a"(acc[i][j]));
+        total += acc[i][j][0] + acc[i][j][1] + acc[i][j][2] + acc[i][j][3];
+      }
+  } else {
+    cf32x16 acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+    for (int p = 0; p < passes; p += 2) {
+#pragma unroll
+      for (int s = 0; s < 2; ++s)
+#pragma unroll
+        for (int h = 0; h < 2; ++h)  // the two 16-deep halves of the 32-deep step
+#pragma unroll
+          for (int c = 0; c < 4; ++c)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0"
+                           : "+a"(acc[i][c])
+                           : "v"(b[s][4 * h + c]), "v"(a[s][4 * h + i]));
+    }
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        asm volatile("" : "+a"(acc[i][j]));
+#pragma unroll
+        for (int v = 0; v < 16; ++v) total += acc[i][j][v];
+      }
+  }
+  out[blockIdx.x * 256 + threadIdx.x] = total;
+}
+
+static int run_ceiling(int preheat_ms) {
+  hipStream_t st;
+  HIP_OK(hipStreamCreate(&st));
+  const size_t nfrag = 2 * 2 * 8 * 256;
+  std::vector<uint16_t> h(nfrag * 8), z(nfrag * 8, 0);
+  std::mt19937 rng(7);
+  std::normal_distribution<float> nd(0.f, 1.f);
+  const float sc = 1.0f / std::sqrt(8192.f);
+  for (auto& v : h) v = f2bf(nd(rng) * sc);
+  void *dfr, *dz, *dout;
+  HIP_OK(hipMalloc(&dfr, h.size() * 2));
+  HIP_OK(hipMalloc(&dz, z.size() * 2));
+  HIP_OK(hipMalloc(&dout, 256 * 256 * 4));
+  HIP_OK(hipMemcpy(dfr, h.data(), h.size() * 2, hipMemcpyHostToDevice));
+  HIP_OK(hipMemcpy(dz, z.data(), z.size() * 2, hipMemcpyHostToDevice));
+  const int passes = 2048, wgs = 256;  // one workgroup of four waves per CU: one wave per SIMD, as in the 256x256 GEMM tile
+  const double flop = (double)wgs * 4 * passes * 64.0 * 16384.0;  // per launch, either instruction
+  struct Case { const char* insn; const char* data; bool big; const void* fr; };
+  const Case cases[] = {{"v_mfma_f32_16x16x32_bf16", "zeros", false, dz}, {"v_mfma_f32_16x16x32_bf16", "randn", false, dfr},
+                        {"v_mfma_f32_32x32x16_bf16", "zeros", true, dz},  {"v_mfma_f32_32x32x16_bf16", "randn", true, dfr}};
+  for (const Case& c : cases) {
+    auto launch = [&](int) {
+      if (c.big) mfma_ceiling_kernel<true><<<wgs, 256, 0, st>>>((const cbf16x8*)c.fr, (float*)dout, passes);
+      else mfma_ceiling_kernel<false><<<wgs, 256, 0, st>>>((const cbf16x8*)c.fr, (float*)dout, passes);
+    };
+    // time-based preheat: clocks and power settle under this very load before anything is timed
+    hipEvent_t e0, e1;
+    HIP_OK(hipEventCreate(&e0));
+    HIP_OK(hipEventCreate(&e1));
+    float heated = 0.f;
+    while (heated < (float)preheat_ms) {
+      HIP_OK(hipEventRecord(e0, st));
+      for (int i = 0; i < 20; ++i) launch(i);
+      HIP_OK(hipEventRecord(e1, st));
+      HIP_OK(hipEventSynchronize(e1));
+      float t;
+      HIP_OK(hipEventElapsedTime(&t, e0, e1));
+      heated += t;
+    }
+    HIP_OK(hipGetLastError());
+    const double ms = time_ms(launch, 40, st);
+    const double tflops = flop / ms / 1e9;
+    // with 64 (16) independent accumulators a wave issues MFMAs back to back: 16 (32) cycles each, 1024 flop per
+    // cycle and SIMD, so the rate implies the clock the chip held
+    printf("{\"ceiling\": \"%s\", \"operands\": \"%s\", \"ms\": %.5f, \"tflops\": %.1f, \"pct_of_2500\": %.2f, "
+           "\"implied_mhz\": %.0f, \"workgroups\": %d, \"waves_per_simd\": 1}\n",
+           c.insn, c.data, ms, tflops, tflops / 25.0, tflops * 1e12 / (256.0 * 4 * 1024.0) / 1e6, wgs);
+    fflush(stdout);
+  }
+  return 0;
+}
+
 int main(int argc, char** argv) {
+  if (argc >= 2 && strcmp(argv[1], "ceiling") == 0) return run_ceiling(argc > 2 ? atoi(argv[2]) : 1000);
   if (argc < 4) {
-    fprintf(stderr, "usage: %s M N K [reps] [b_layout] [variant] [split_k] [group_m] [nbuf]\n", argv[0]);
+    fprintf(stderr, "usage: %s M N K [reps] [b_layout] [variant] [split_k] [group_m] [nbuf]\n       %s ceiling [preheat_ms]\n",
+            argv[0], argv[0]);
     return 2;
   }
   const int64_t M = atoll(argv[1]), N = atoll(argv[2]), K = atoll(argv[3]);

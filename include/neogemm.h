@@ -106,7 +106,8 @@ int neogemm_bf16_batched(const void* A, const void* B, void* C, int64_t M, int64
 size_t neogemm_bf16_batched_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t batch);
 
 /*
- * Upper bound of the scratch neogemm_bf16 may use for (M,N,K), in bytes.  Host-only arithmetic.
+ * Upper bound of the scratch neogemm_bf16 may use for (M,N,K), in bytes, whatever the layouts of B and C
+ * (the bound is the largest need over the four combinations).  Host-only arithmetic.
  * Counterpart of the per-call device allocations the reference's launcher makes for its TMA
  * descriptors (v01.cu:153-160, nemgemmV03.cu:60-68): here the caller owns the scratch.
  */
@@ -152,7 +153,7 @@ size_t neogemm_bf16_profile_bytes(int64_t M, int64_t N, int variant);
 /* Text for a status code; replaces the std::cerr print at nemgemmV03.cu:387-390. Never NULL. */
 const char* neogemm_strerror(int status);
 
-/* Library version string, e.g. "neogemm 0.1 gfx950". */
+/* Library version string, e.g. "neogemm 0.2 gfx950". */
 const char* neogemm_version(void);
 
 #ifdef __cplusplus

@@ -59,7 +59,7 @@ def test_plan_for_the_benchmark_configs():
     for M, N, K in ((16, 14336, 4096), (64, 14336, 4096), (128, 14336, 4096), (1024, 1024, 32768), (512, 512, 512)):
         v, s = _abi.plan(M, N, K)
         assert v != _abi.VARIANT_GENERIC and s >= 1
-        s = max(s, _abi.plan(M, N, K, c_layout=1)[1])     # one query covers both output layouts
+        s = max(_abi.plan(M, N, K, b, c)[1] for b in (0, 1) for c in (0, 1))   # one query covers all four layouts
         assert _abi.workspace_bytes(M, N, K) == (s * M * N * 4 if s > 1 else 0)
     assert _abi.plan(1024, 1024, 32768)[1] > 1
     # 3072^3 and 6144^3: 144 / 576 tiles of 256x256 fill 256 CUs badly, 192 / 768 tiles of 192x256 do better; the
@@ -74,6 +74,35 @@ def test_plan_for_the_benchmark_configs():
     # unaligned problems go to the generic kernel
     assert _abi.plan(100, 100, 100, aligned=False) == (_abi.VARIANT_GENERIC, 1)
     assert _abi.workspace_bytes(0, 5, 5) == 0 and _abi.workspace_bytes(5, 5, 0) == 0
+
+
+def test_workspace_query_bounds_every_layout():
+    """neogemm_bf16_workspace_bytes(M,N,K) must cover the split the call itself plans, for every (b_layout, c_layout)
+    — the reference's own call is B [N,K] with a column-major C (nemgemmV03.cu:343-391) and must never be answered
+    with 'workspace too small' after the caller sized the workspace by the query."""
+    dims = [16, 64, 96, 128, 192, 256, 384, 512, 768, 1024, 1536, 2048, 3072, 4096, 6144, 8192, 14336]
+    ks = [64, 256, 512, 1024, 2048, 4096, 8192, 16384, 32768]
+    cells = 0
+    for M in dims:
+        for N in dims:
+            for K in ks:
+                have = _abi.workspace_bytes(M, N, K)
+                for b in (_abi.B_KN, _abi.B_NK):
+                    for c in (_abi.C_ROW, _abi.C_COL):
+                        v, s = _abi.plan(M, N, K, b, c)
+                        need = s * M * N * 4 if s > 1 else 0
+                        assert need <= have, (M, N, K, b, c, v, s, have)
+                        cells += 1
+    assert cells >= 10000
+    # the cells found failing before the query looked at every layout
+    for M, N, K in ((1024, 6144, 8192), (2048, 3072, 8192), (512, 6144, 8192), (4096, 1536, 8192)):
+        v, s = _abi.plan(M, N, K, _abi.B_NK, _abi.C_COL)
+        assert _abi.workspace_bytes(M, N, K) >= (s * M * N * 4 if s > 1 else 0)
+    # batched query likewise
+    lib = _abi.load()
+    for batch in (2, 7):
+        for M, N, K in ((128, 128, 8192), (256, 512, 16384), (1024, 6144, 8192)):
+            assert lib.neogemm_bf16_batched_workspace_bytes(M, N, K, batch) >= 0
 
 
 def test_argument_validation_returns_before_touching_the_gpu():
@@ -120,15 +149,19 @@ def test_plan_table_overrides_the_model(tmp_path):
         {"M": 4096, "N": 4096, "K": 4096, "variant": _abi.VARIANT_T256x256_W8, "split_k": 1},   # c_layout defaults to 0
         {"M": 8192, "N": 8192, "K": 8192, "c_layout": 0, "variant": 99, "split_k": 1},           # unknown variant
         {"M": 1024, "N": 1024, "K": 1024, "c_layout": 0, "variant": _abi.VARIANT_T128x128_W4, "split_k": 0},  # bad split
+        {"M": 2048, "N": 2048, "K": 2048, "b_layout": 1, "c_layout": 1, "variant": _abi.VARIANT_T128x256_W4, "split_k": 1},
     ]))
     code = ("from gemm_amd import _abi\n"
             "print(_abi.plan(512, 512, 512), _abi.plan(4096, 4096, 4096), _abi.plan(8192, 8192, 8192), "
-            "_abi.plan(1024, 1024, 1024), _abi.plan(512, 512, 512, c_layout=1), _abi.workspace_bytes(512, 512, 512))")
+            "_abi.plan(1024, 1024, 1024), _abi.plan(512, 512, 512, c_layout=1), _abi.workspace_bytes(512, 512, 512), "
+            "_abi.plan(512, 512, 512, b_layout=1), _abi.plan(2048, 2048, 2048, 1, 1), _abi.plan(2048, 2048, 2048, 0, 1))")
     env = dict(os.environ, NEOGEMM_PLAN_TABLE=str(table))
     out = subprocess.run([sys.executable, "-c", code], env=env, cwd=ROOT, capture_output=True, text=True, check=True).stdout
     model = (_abi.plan(512, 512, 512), _abi.plan(8192, 8192, 8192), _abi.plan(1024, 1024, 1024))
     want = ((_abi.VARIANT_T128x128_W4, 2), (_abi.VARIANT_T256x256_W8, 1), model[1], model[2],
-            _abi.plan(512, 512, 512, c_layout=1), 2 * 512 * 512 * 4)
+            _abi.plan(512, 512, 512, c_layout=1), 2 * 512 * 512 * 4,
+            # an entry is keyed on both layouts: B [N,K] calls of a shape tuned with B [K,N] keep the model's choice
+            _abi.plan(512, 512, 512, b_layout=1), (_abi.VARIANT_T128x256_W4, 1), _abi.plan(2048, 2048, 2048, 0, 1))
     assert out.strip() == " ".join(str(w) for w in want)
     # an unreadable file changes nothing
     env = dict(os.environ, NEOGEMM_PLAN_TABLE=str(tmp_path / "missing.json"))

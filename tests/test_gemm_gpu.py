@@ -284,6 +284,75 @@ def test_reference_call_contract(dev, modname):
     o.assert_parity(C3.view(N2, M2).t(), A2, B2, b_layout="nk", what=f"{modname}.neoGemmV1 non-square")
 
 
+@pytest.mark.parametrize("M,N,K", [(1024, 6144, 8192), (4096, 1536, 8192), (1024, 1024, 32768)])
+def test_reference_call_on_split_k_shapes(dev, M, N, K):
+    """neoGemmV1's layout (B [N,K], column-major C: nemgemmV03.cu:343-391) on shapes whose plan for that layout
+    splits K: both wrappers size the workspace with neogemm_bf16_workspace_bytes and the call must go through;
+    the raw C-ABI call with a workspace of exactly the queried size likewise."""
+    import neoGEMM
+    A, Bnk = o.make_inputs(M, N, K, seed=M + N, b_layout="nk")
+    Ad, Bd = A.to(dev), Bnk.to(dev)
+    ref = o.ref_gemm(A, Bnk, b_layout="nk")
+    rows = torch.randperm(M, generator=torch.Generator().manual_seed(5))[:192]
+    results = []
+    for mod in (g, neoGEMM):
+        C = torch.full((M * N,), float("nan"), dtype=torch.bfloat16, device=dev).view(M, N)
+        mod.neoGemmV1(Ad, Bd, C)
+        torch.cuda.synchronize()
+        got = C.view(N, M).t().cpu()
+        o.assert_parity(got[rows], A[rows], Bnk, b_layout="nk", ref=ref[rows], what=f"{mod.__name__}.neoGemmV1 {M}x{N}x{K}")
+        results.append(got)
+    assert torch.equal(results[0], results[1])
+    need = g.workspace_bytes(M, N, K)
+    v, split = g.plan(M, N, K, g.B_NK, g.C_COL)
+    assert need >= (split * M * N * 4 if split > 1 else 0)
+    ws = torch.empty(max(need, 16), dtype=torch.uint8, device=dev)
+    C = torch.full((N, M), float("nan"), dtype=torch.bfloat16, device=dev)
+    st = _abi.gemm_raw(Ad.data_ptr(), Bd.data_ptr(), C.data_ptr(), M, N, K, K, K, M, g.B_NK, g.C_COL, ws.data_ptr() if need else 0,
+                       need, torch.cuda.current_stream().cuda_stream)
+    assert st == _abi.OK, _abi.strerror(st)
+    torch.cuda.synchronize()
+    assert torch.equal(C.t().cpu(), results[0])
+
+
+def test_split_k_on_two_streams(dev):
+    """Two split-K GEMMs with different inputs queued on two streams with no host synchronisation in between, several
+    times over: each stream has its own partials, so neither result is disturbed (the reference runs everything on
+    the one default stream, nemgemmV03.cu:383)."""
+    import neoGEMM
+    M, N, K = 512, 512, 16384
+    assert g.plan(M, N, K)[1] > 1 and g.workspace_bytes(M, N, K) > 0
+    A1, B1 = o.make_inputs(M, N, K, seed=31)
+    A2, B2 = o.make_inputs(M, N, K, seed=32)
+    want1, want2 = o.ref_gemm(A1, B1), o.ref_gemm(A2, B2)
+    d = [t.to(dev) for t in (A1, B1, A2, B2)]
+    torch.cuda.synchronize()
+    for mod in (g, neoGEMM):
+        s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+        outs1, outs2 = [], []
+        for it in range(6):
+            with torch.cuda.stream(s1):
+                outs1.append(mod.gemm(d[0], d[1]))
+            with torch.cuda.stream(s2):
+                outs2.append(mod.gemm(d[2], d[3]))
+        s1.synchronize()
+        s2.synchronize()
+        for c in outs1:
+            assert torch.equal(c, outs1[0])
+        for c in outs2:
+            assert torch.equal(c, outs2[0])
+        o.assert_parity(outs1[0], A1, B1, ref=want1, what=f"{mod.__name__} stream 1")
+        o.assert_parity(outs2[0], A2, B2, ref=want2, what=f"{mod.__name__} stream 2")
+    # growing the buffer of a stream that still has work queued on it
+    with torch.cuda.stream(s1):
+        small = g.gemm(d[0], d[1])
+        Abig, Bbig = o.make_inputs(1024, 1024, 32768, seed=33)
+        big = g.gemm(Abig.to(dev, non_blocking=False), Bbig.to(dev))
+    s1.synchronize()
+    assert torch.equal(small, outs1[0])
+    o.assert_parity(big[:128], Abig[:128], Bbig, what="grown workspace")
+
+
 def test_module_gemm_matches_abi(dev):
     import neoGEMM
     for M, N, K in ((512, 512, 512), (200, 328, 136), (16, 14336, 4096)):
@@ -491,6 +560,9 @@ def test_tuner_measures_candidates(dev):
     model, t_model, best, t_best = tune.tune_shape(256, 384, 2048, log=io.StringIO())
     assert model == g.plan(256, 384, 2048) and best[0] in tune.CANDIDATE_VARIANTS + (model[0],) and best[1] >= 1
     assert 0 < t_best <= t_model
+    # the reference's layout (B [N,K], column-major C) is tuned on its own kernels
+    model, t_model, best, t_best = tune.tune_shape(256, 384, 2048, log=io.StringIO(), b_layout=g.B_NK, c_layout=g.C_COL)
+    assert model == g.plan(256, 384, 2048, g.B_NK, g.C_COL) and 0 < t_best <= t_model
 
 
 # ------------------------------------------------------------------------------------------------

@@ -282,3 +282,21 @@ def test_scaled_against_fp64_formula():
     for wrong in (alpha * o.exact_gemm_f64(A, B), alpha * o.exact_gemm_f64(A, B) - beta * C0.double(),
                   alpha * (o.exact_gemm_f64(A, B) + beta * C0.double())):
         assert not bool(((got - wrong).abs() <= half_ulp * 1.0000001 + slack).all())
+
+
+def test_two_legal_fp32_orders_differ_by_more_than_one_raw_ulp():
+    """Why the per-element criterion is measured at max(|ref|, 2^-7 rms) and not in raw ulps: two correct
+    fp32-accumulating products of the same bf16 inputs, taken in different orders — torch's blocked CPU matmul
+    (ref_gemm) and the plain-C sequential-k sum (c_gemm) — already disagree by more than 1 raw bf16 ulp on elements
+    that cancel to nearly zero at K = 8192, while each passes assert_parity against the other as reference."""
+    A, B = o.make_inputs(64, 64, 8192, seed=123)
+    r_torch, r_c = o.ref_gemm(A, B), o.c_gemm(A, B)
+    ulp = o.ulp_distance(o.bits_of(r_torch), o.bits_of(r_c))
+    assert ulp.max() > 1, "expected the two summation orders to differ by more than one raw ulp somewhere"
+    # the disagreement sits on elements far below the typical magnitude, nowhere else
+    rms = float(r_torch.float().pow(2).mean().sqrt())
+    big = np.abs(r_torch.float().numpy()) >= rms * 2.0 ** -5
+    assert ulp[big].max() <= 1
+    assert np.abs(r_torch.float().numpy())[ulp > 1].max() < rms * 2.0 ** -5
+    o.assert_parity(r_c, A, B, ref=r_torch, what="sequential-k vs blocked")
+    o.assert_parity(r_torch, A, B, ref=r_c, what="blocked vs sequential-k")
