@@ -21,6 +21,17 @@
 
 #include "neogemm.h"
 
+// Split build: compiling this one file takes minutes because of the many instances of the tile kernel, so setup.py
+// compiles it NEOGEMM_PARTS times in parallel with -DNEOGEMM_PART=0..NEOGEMM_PARTS-1 and links the objects.  Part 0
+// holds everything but the tile kernels; part k > 0 instantiates its share of launch_tile<> (listed behind
+// launch_tile) and nothing else.  Without NEOGEMM_PART the file is one self-contained translation unit.
+#ifdef NEOGEMM_PART
+#define NEOGEMM_HAS_PART(p) (NEOGEMM_PART == (p))
+#else
+#define NEOGEMM_HAS_PART(p) 1
+#endif
+#define NEOGEMM_PARTS 7
+
 namespace neogemm {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
@@ -758,6 +769,108 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
   }
 }
 
+// Raise a kernel's dynamic-LDS limit once per (instantiation, device): the attribute belongs to the current
+// device's copy of the function.  `done` holds one bit per device index.
+template <class Kern>
+static hipError_t allow_lds(Kern kern, size_t lds, std::atomic<uint64_t>& done) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  const uint64_t bit = 1ull << (dev & 63);
+  if (dev > 63 || !(done.load(std::memory_order_acquire) & bit)) {
+    e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return e;
+    done.fetch_or(bit, std::memory_order_release);
+  }
+  return hipSuccess;
+}
+
+template <int BM, int BN, int WGM, int WGN>
+hipError_t launch_tile(const TileArgs& a, bool ak, bool bk, hipStream_t st) {
+  // A: three 64-deep images if K-major, else four 32-deep ones; B likewise, but two or three 64-deep ones if both are K-major
+  size_t lds = (size_t)BM * (ak ? 384 : 256) + (size_t)BN * (bk ? (ak ? b_images_both_kmajor(BM, BN) * 128 : 384) : 256);
+  dim3 grid(a.ntm * a.ntn, a.ksplit, a.batch), block(WGM * WGN * 64);
+  auto go = [&](auto kern) -> hipError_t {
+    static std::atomic<uint64_t> attr_done{0};  // per instantiation
+    if (hipError_t e = allow_lds(kern, lds, attr_done); e != hipSuccess) return e;
+    kern<<<grid, block, lds, st>>>(a);
+    return hipGetLastError();
+  };
+  if (a.prof) {
+    if constexpr (BM == 256 && BN == 256) {
+      if (ak && bk) return go(gemm_tile_kernel<BM, BN, WGM, WGN, true, true, true>);
+      if (ak && !bk) return go(gemm_tile_kernel<BM, BN, WGM, WGN, true, false, true>);
+    }
+    return hipErrorInvalidValue;
+  }
+  if (ak && bk) {
+    if constexpr (BM == 128 && BN == 128) {
+      // more workgroups than CUs: two images of B, 80 KiB, so that two workgroups share a CU
+      if ((int64_t)a.ntm * a.ntn * a.ksplit * a.batch > 256) {
+        lds = (size_t)BM * 384 + (size_t)BN * 256;
+        return go(gemm_tile_kernel<BM, BN, WGM, WGN, true, true, false, 2>);
+      }
+    }
+    return go(gemm_tile_kernel<BM, BN, WGM, WGN, true, true>);
+  }
+  if (ak && !bk) {
+    if constexpr (BN >= 128 && (BN & (BN - 1)) == 0) return go(gemm_tile_kernel<BM, BN, WGM, WGN, true, false>);
+  }
+  if (!ak && bk) {
+    if constexpr (BM >= 128 && (BM & (BM - 1)) == 0) return go(gemm_tile_kernel<BM, BN, WGM, WGN, false, true>);
+  }
+  return hipErrorInvalidValue;
+}
+
+// The tile kernels are instantiated through launch_tile.  In a split build each part instantiates its share and
+// the others only declare it.
+#ifdef NEOGEMM_PART
+#define NEOGEMM_TILE(BM, BN, WGM, WGN) \
+  template hipError_t launch_tile<BM, BN, WGM, WGN>(const TileArgs&, bool, bool, hipStream_t);
+#if NEOGEMM_PART == 1
+NEOGEMM_TILE(256, 256, 2, 2)
+#else
+extern NEOGEMM_TILE(256, 256, 2, 2)
+#endif
+#if NEOGEMM_PART == 2
+NEOGEMM_TILE(256, 256, 2, 4)
+NEOGEMM_TILE(64, 128, 1, 4)
+#else
+extern NEOGEMM_TILE(256, 256, 2, 4)
+extern NEOGEMM_TILE(64, 128, 1, 4)
+#endif
+#if NEOGEMM_PART == 3
+NEOGEMM_TILE(128, 128, 2, 2)
+NEOGEMM_TILE(128, 128, 1, 4)
+#else
+extern NEOGEMM_TILE(128, 128, 2, 2)
+extern NEOGEMM_TILE(128, 128, 1, 4)
+#endif
+#if NEOGEMM_PART == 4
+NEOGEMM_TILE(256, 128, 2, 2)
+#else
+extern NEOGEMM_TILE(256, 128, 2, 2)
+#endif
+#if NEOGEMM_PART == 5
+NEOGEMM_TILE(128, 256, 2, 2)
+#else
+extern NEOGEMM_TILE(128, 256, 2, 2)
+#endif
+#if NEOGEMM_PART == 6
+NEOGEMM_TILE(192, 256, 2, 2)
+#else
+extern NEOGEMM_TILE(192, 256, 2, 2)
+#endif
+#undef NEOGEMM_TILE
+#endif
+
+}  // namespace neogemm
+
+// Everything below — the other kernels, the planner, the launcher and the C ABI — belongs to part 0 of a
+// split build (see NEOGEMM_PART at the top of the file).
+#if NEOGEMM_HAS_PART(0)
+namespace neogemm {
+
 // ---------------------------------------------------------------------------------------------
 // Skinny M (decode shapes: M <= 16 * TMF; C row-major or, CCOL, column-major): bound by streaming B from HBM once, so what
 // counts is bytes in flight per CU, not MFMA rate.  A workgroup owns a strip of 64 columns of C and the
@@ -1056,59 +1169,6 @@ static const VariantInfo kVariants[NEOGEMM_VARIANT_COUNT] = {
     {0, 0, 0}, {16, 16, 4}, {256, 256, 8}, {256, 256, 4}, {128, 128, 4}, {256, 128, 4}, {128, 256, 4}, {64, 128, 4}, {128, 128, 4},
     {16, 64, 4}, {32, 64, 4}, {64, 64, 4}, {192, 256, 4},
 };
-
-// Raise a kernel's dynamic-LDS limit once per (instantiation, device): the attribute belongs to the current
-// device's copy of the function.  `done` holds one bit per device index.
-template <class Kern>
-static hipError_t allow_lds(Kern kern, size_t lds, std::atomic<uint64_t>& done) {
-  int dev = 0;
-  hipError_t e = hipGetDevice(&dev);
-  if (e != hipSuccess) return e;
-  const uint64_t bit = 1ull << (dev & 63);
-  if (dev > 63 || !(done.load(std::memory_order_acquire) & bit)) {
-    e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return e;
-    done.fetch_or(bit, std::memory_order_release);
-  }
-  return hipSuccess;
-}
-
-template <int BM, int BN, int WGM, int WGN>
-static hipError_t launch_tile(const TileArgs& a, bool ak, bool bk, hipStream_t st) {
-  // A: three 64-deep images if K-major, else four 32-deep ones; B likewise, but two or three 64-deep ones if both are K-major
-  size_t lds = (size_t)BM * (ak ? 384 : 256) + (size_t)BN * (bk ? (ak ? b_images_both_kmajor(BM, BN) * 128 : 384) : 256);
-  dim3 grid(a.ntm * a.ntn, a.ksplit, a.batch), block(WGM * WGN * 64);
-  auto go = [&](auto kern) -> hipError_t {
-    static std::atomic<uint64_t> attr_done{0};  // per instantiation
-    if (hipError_t e = allow_lds(kern, lds, attr_done); e != hipSuccess) return e;
-    kern<<<grid, block, lds, st>>>(a);
-    return hipGetLastError();
-  };
-  if (a.prof) {
-    if constexpr (BM == 256 && BN == 256) {
-      if (ak && bk) return go(gemm_tile_kernel<BM, BN, WGM, WGN, true, true, true>);
-      if (ak && !bk) return go(gemm_tile_kernel<BM, BN, WGM, WGN, true, false, true>);
-    }
-    return hipErrorInvalidValue;
-  }
-  if (ak && bk) {
-    if constexpr (BM == 128 && BN == 128) {
-      // more workgroups than CUs: two images of B, 80 KiB, so that two workgroups share a CU
-      if ((int64_t)a.ntm * a.ntn * a.ksplit * a.batch > 256) {
-        lds = (size_t)BM * 384 + (size_t)BN * 256;
-        return go(gemm_tile_kernel<BM, BN, WGM, WGN, true, true, false, 2>);
-      }
-    }
-    return go(gemm_tile_kernel<BM, BN, WGM, WGN, true, true>);
-  }
-  if (ak && !bk) {
-    if constexpr (BN >= 128 && (BN & (BN - 1)) == 0) return go(gemm_tile_kernel<BM, BN, WGM, WGN, true, false>);
-  }
-  if (!ak && bk) {
-    if constexpr (BM >= 128 && (BM & (BM - 1)) == 0) return go(gemm_tile_kernel<BM, BN, WGM, WGN, false, true>);
-  }
-  return hipErrorInvalidValue;
-}
 
 static bool is_aligned(const void* A, const void* B, const void* C, int64_t K, int64_t lda, int64_t ldb,
                        int64_t ldc) {
@@ -1555,6 +1615,8 @@ const char* neogemm_strerror(int status) {
   }
 }
 
-const char* neogemm_version(void) { return "neogemm 0.1 gfx950"; }
+const char* neogemm_version(void) { return "neogemm 0.2 gfx950"; }
 
 }  // extern "C"
+
+#endif  // NEOGEMM_HAS_PART(0)

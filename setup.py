@@ -18,16 +18,37 @@ ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 LIB = os.path.join(ROOT, "gemm_amd", "libneogemm.so")
 
 HIPCC_FLAGS = [
-    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-DNDEBUG",
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-DNDEBUG",
     # packed-fp32 VALU forms are kept off for every HIP file of this project
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
+KERNEL_PARTS = 7  # NEOGEMM_PARTS in gemm_amd/csrc/neogemm.hip
 
 
 def build_kernels():
-    """hipcc -> gemm_amd/libneogemm.so (cross-compiles without a GPU)."""
+    """hipcc -> gemm_amd/libneogemm.so (cross-compiles without a GPU).
+
+    The one source file is compiled KERNEL_PARTS times in parallel, each time with a different share of the tile
+    kernel's instances (-DNEOGEMM_PART=k), and the objects are linked into the library.
+    """
+    from concurrent.futures import ThreadPoolExecutor
+
+    hipcc = os.path.join(ROCM, "bin", "hipcc")
     src = os.path.join(ROOT, "gemm_amd", "csrc", "neogemm.hip")
-    cmd = [os.path.join(ROCM, "bin", "hipcc"), *HIPCC_FLAGS, "-I", os.path.join(ROOT, "include"), "-o", LIB, src]
+    objdir = os.path.join(ROOT, "build", "neogemm_parts")
+    os.makedirs(objdir, exist_ok=True)
+
+    def compile_part(k):
+        obj = os.path.join(objdir, f"neogemm_part{k}.o")
+        cmd = [hipcc, *HIPCC_FLAGS, f"-DNEOGEMM_PART={k}", "-I", os.path.join(ROOT, "include"), "-c", "-o", obj, src]
+        print(" ".join(cmd), flush=True)
+        subprocess.check_call(cmd)
+        return obj
+
+    jobs = max(1, min(KERNEL_PARTS, int(os.environ.get("MAX_JOBS", os.cpu_count() or 1))))
+    with ThreadPoolExecutor(max_workers=jobs) as pool:
+        objs = list(pool.map(compile_part, range(KERNEL_PARTS)))
+    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]
     print(" ".join(cmd), flush=True)
     subprocess.check_call(cmd)
 
