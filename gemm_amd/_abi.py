@@ -9,7 +9,8 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libneogemm.so")
 
-OK, ERR_BAD_ARG, ERR_WORKSPACE, ERR_UNSUPPORTED, ERR_LAUNCH = 0, -1, -2, -3, -4
+OK, ERR_BAD_ARG, ERR_WORKSPACE, ERR_UNSUPPORTED, ERR_LAUNCH, ERR_SCRATCH_LIMIT = 0, -1, -2, -3, -4, -5
+NOALLOC_SCRATCH_BYTES = 32 * 1024 * 1024
 B_KN, B_NK = 0, 1
 C_ROW, C_COL = 0, 1
 VARIANT_AUTO, VARIANT_GENERIC = 0, 1
@@ -26,6 +27,7 @@ VARIANT_NAMES = {0: "auto", 1: "generic", 2: "256x256_w8", 3: "256x256_w4", 4: "
 _i64, _int, _vp, _sz = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t
 PROTOTYPES = {
     "neogemm_bf16": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _vp, _sz, _vp]),
+    "neogemm_bf16_noalloc": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _vp]),
     "neogemm_bf16_scaled": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, ctypes.c_float,
                                    ctypes.c_float, _vp, _sz, _vp]),
     "neogemm_bf16_batched": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int,

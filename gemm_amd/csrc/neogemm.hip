@@ -1529,9 +1529,49 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
   return NEOGEMM_OK;
 }
 
+// Split-K partials of the entry point that allocates nothing (neogemm_bf16_noalloc): one array per GPU, laid out
+// by the code object, held until the process ends.  In host code the name `scratch` only stands for the symbol;
+// the device address is asked for once per device (scratch_on_current_device) and that pointer is what the kernels get.
+static __device__ __align__(256) unsigned char scratch[NEOGEMM_NOALLOC_SCRATCH_BYTES];
+
+static int scratch_on_current_device(void** out) {
+  static std::mutex mu;
+  static void* ptrs[64] = {};
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return NEOGEMM_ERR_LAUNCH;
+  std::lock_guard<std::mutex> lock(mu);
+  if (!ptrs[dev]) {
+    void* p = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) {
+      fprintf(stderr, "neogemm: hipGetSymbolAddress(scratch) failed on device %d: %s\n", dev, hipGetErrorString(e));
+      return NEOGEMM_ERR_LAUNCH;
+    }
+    ptrs[dev] = p;
+  }
+  *out = ptrs[dev];
+  return NEOGEMM_OK;
+}
+
 }  // namespace neogemm
 
 extern "C" {
+
+int neogemm_bf16_noalloc(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int64_t lda,
+                         int64_t ldb, int64_t ldc, int b_layout, int c_layout, void* hip_stream) {
+  // what neogemm_bf16 would be handed as a workspace for this shape, taken from the built-in array instead
+  size_t need = 0;
+  if (M > 0 && N > 0 && K > 0 && M <= 0x7fffffff && N <= 0x7fffffff && K <= 0x7fffffff)
+    need = neogemm_bf16_workspace_bytes(M, N, K);
+  if (need > (size_t)NEOGEMM_NOALLOC_SCRATCH_BYTES) return NEOGEMM_ERR_SCRATCH_LIMIT;
+  void* ws = nullptr;
+  if (need) {
+    const int st = neogemm::scratch_on_current_device(&ws);
+    if (st != NEOGEMM_OK) return st;
+  }
+  return neogemm::run(A, B, C, M, N, K, lda, ldb, ldc, b_layout, c_layout, ws, need, hip_stream, NEOGEMM_VARIANT_AUTO, 0,
+                      0);
+}
 
 int neogemm_bf16(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
                  int64_t ldc, int b_layout, int c_layout, void* workspace, size_t workspace_bytes, void* hip_stream) {
@@ -1611,6 +1651,9 @@ const char* neogemm_strerror(int status) {
     case NEOGEMM_ERR_WORKSPACE: return "workspace missing or too small (see neogemm_bf16_workspace_bytes)";
     case NEOGEMM_ERR_UNSUPPORTED: return "the requested kernel variant cannot run this shape or alignment";
     case NEOGEMM_ERR_LAUNCH: return "HIP kernel launch failed";
+    case NEOGEMM_ERR_SCRATCH_LIMIT:
+      return "the shape needs more split-K scratch than the built-in NEOGEMM_NOALLOC_SCRATCH_BYTES (32 MiB): "
+             "call neogemm_bf16 with a workspace instead";
     default: return "unknown neogemm status";
   }
 }

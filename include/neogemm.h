@@ -30,6 +30,7 @@ extern "C" {
 #define NEOGEMM_ERR_WORKSPACE (-2)    /* workspace missing or smaller than neogemm_bf16_workspace_bytes */
 #define NEOGEMM_ERR_UNSUPPORTED (-3)  /* the forced variant cannot run this shape / alignment */
 #define NEOGEMM_ERR_LAUNCH (-4)       /* HIP refused the launch (see stderr for hipGetErrorString) */
+#define NEOGEMM_ERR_SCRATCH_LIMIT (-5) /* neogemm_bf16_noalloc: the shape needs more than NEOGEMM_NOALLOC_SCRATCH_BYTES */
 
 /* b_layout values */
 #define NEOGEMM_B_KN 0 /* B is [K,N] row-major (N contiguous): the layout `C = gemm(A, B)` is quoted on */
@@ -104,6 +105,21 @@ int neogemm_bf16_batched(const void* A, const void* B, void* C, int64_t M, int64
                          int64_t batch, int b_layout, int c_layout, void* workspace, size_t workspace_bytes,
                          void* hip_stream);
 size_t neogemm_bf16_batched_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t batch);
+
+/*
+ * neogemm_bf16 for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same arguments and
+ * result as neogemm_bf16 (bit for bit: the same kernels run), minus the workspace: split-K partials go to
+ * an array of NEOGEMM_NOALLOC_SCRATCH_BYTES that the library's code object holds on each GPU it runs on,
+ * until the process ends.  The call makes no hipMalloc/hipFree and no other allocating call.  A shape whose
+ * neogemm_bf16_workspace_bytes(M,N,K) exceeds NEOGEMM_NOALLOC_SCRATCH_BYTES is refused with
+ * NEOGEMM_ERR_SCRATCH_LIMIT and nothing is launched.  All calls on one GPU share that GPU's array: calls on
+ * one stream are ordered and safe (every partial is rewritten before it is read, nothing has to start at
+ * zero); calls that overlap in time on one GPU (different streams or threads) race on it.
+ */
+#define NEOGEMM_NOALLOC_SCRATCH_BYTES (32u * 1024u * 1024u)
+int neogemm_bf16_noalloc(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int64_t lda,
+                         int64_t ldb, int64_t ldc, int b_layout, int c_layout, void* hip_stream);
 
 /*
  * Upper bound of the scratch neogemm_bf16 may use for (M,N,K), in bytes, whatever the layouts of B and C
