@@ -12,7 +12,7 @@
 #include <stdio.h>
 #include <stdlib.h>
 
-#include <atomic>
+#include <map>
 #include <mutex>
 #include <type_traits>
 #include <string>
@@ -30,7 +30,7 @@
 #else
 #define NEOGEMM_HAS_PART(p) 1
 #endif
-#define NEOGEMM_PARTS 7
+#define NEOGEMM_PARTS 8
 
 namespace neogemm {
 
@@ -769,18 +769,22 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
   }
 }
 
-// Raise a kernel's dynamic-LDS limit once per (instantiation, device): the attribute belongs to the current
-// device's copy of the function.  `done` holds one bit per device index.
+// Raise a kernel's dynamic-LDS limit once per (kernel, device): the attribute belongs to the current device's copy
+// of the function.  The registry is keyed on the kernel's address (all instances share one function-pointer type).
 template <class Kern>
-static hipError_t allow_lds(Kern kern, size_t lds, std::atomic<uint64_t>& done) {
+static hipError_t allow_lds(Kern kern, size_t lds) {
+  static std::mutex mu;
+  static std::map<const void*, uint64_t> done;  // kernel -> one bit per device index
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return e;
   const uint64_t bit = 1ull << (dev & 63);
-  if (dev > 63 || !(done.load(std::memory_order_acquire) & bit)) {
+  std::lock_guard<std::mutex> lock(mu);
+  uint64_t& mask = done[(const void*)kern];
+  if (dev > 63 || !(mask & bit)) {
     e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
-    done.fetch_or(bit, std::memory_order_release);
+    mask |= bit;
   }
   return hipSuccess;
 }
@@ -791,8 +795,7 @@ hipError_t launch_tile(const TileArgs& a, bool ak, bool bk, hipStream_t st) {
   size_t lds = (size_t)BM * (ak ? 384 : 256) + (size_t)BN * (bk ? (ak ? b_images_both_kmajor(BM, BN) * 128 : 384) : 256);
   dim3 grid(a.ntm * a.ntn, a.ksplit, a.batch), block(WGM * WGN * 64);
   auto go = [&](auto kern) -> hipError_t {
-    static std::atomic<uint64_t> attr_done{0};  // per instantiation
-    if (hipError_t e = allow_lds(kern, lds, attr_done); e != hipSuccess) return e;
+    if (hipError_t e = allow_lds(kern, lds); e != hipSuccess) return e;
     kern<<<grid, block, lds, st>>>(a);
     return hipGetLastError();
   };
@@ -860,6 +863,13 @@ extern NEOGEMM_TILE(128, 256, 2, 2)
 NEOGEMM_TILE(192, 256, 2, 2)
 #else
 extern NEOGEMM_TILE(192, 256, 2, 2)
+#endif
+#if NEOGEMM_PART == 7
+NEOGEMM_TILE(96, 128, 2, 2)
+NEOGEMM_TILE(64, 64, 2, 2)
+#else
+extern NEOGEMM_TILE(96, 128, 2, 2)
+extern NEOGEMM_TILE(64, 64, 2, 2)
 #endif
 #undef NEOGEMM_TILE
 #endif
@@ -1167,7 +1177,7 @@ struct VariantInfo {
 };
 static const VariantInfo kVariants[NEOGEMM_VARIANT_COUNT] = {
     {0, 0, 0}, {16, 16, 4}, {256, 256, 8}, {256, 256, 4}, {128, 128, 4}, {256, 128, 4}, {128, 256, 4}, {64, 128, 4}, {128, 128, 4},
-    {16, 64, 4}, {32, 64, 4}, {64, 64, 4}, {192, 256, 4},
+    {16, 64, 4}, {32, 64, 4}, {64, 64, 4}, {192, 256, 4}, {96, 128, 4}, {64, 64, 4},
 };
 
 static bool is_aligned(const void* A, const void* B, const void* C, int64_t K, int64_t lda, int64_t ldb,
@@ -1197,6 +1207,7 @@ static const PlanCand kPlanCands[] = {
     {NEOGEMM_VARIANT_T256x256_W4, 1.33, 9.0, 12.0, 1}, {NEOGEMM_VARIANT_T128x256_W4, 0.78, 6.0, 5.0, 1},
     {NEOGEMM_VARIANT_T256x128_W4, 0.78, 6.0, 5.0, 1},  {NEOGEMM_VARIANT_T128x128_W4, 0.50, 3.0, 2.0, 2},
     {NEOGEMM_VARIANT_T64x128_W4, 0.35, 2.5, 1.0, 2},    {NEOGEMM_VARIANT_T192x256_W4, 1.0, 7.0, 9.0, 1},
+    {NEOGEMM_VARIANT_T96x128_W4, 0.42, 2.8, 1.8, 1},    {NEOGEMM_VARIANT_T64x64_W4, 0.20, 2.0, 1.0, 2},
 };
 static void plan_model(int64_t M, int64_t N, int64_t K, bool aligned, int c_layout, int* variant, int* split_k,
                        int64_t batch = 1, int b_layout = NEOGEMM_B_KN) {
@@ -1217,7 +1228,12 @@ static void plan_model(int64_t M, int64_t N, int64_t K, bool aligned, int c_layo
     // the 64x128 tile has too little in flight to stream from HBM: only for problems that stay in cache
     if (c.variant == NEOGEMM_VARIANT_T64x128_W4 && bytes > 32e6) continue;
     // 192 rows only of a K-major operand (an MN-major image needs a power of two)
-    if (c.variant == NEOGEMM_VARIANT_T192x256_W4 && c_layout == NEOGEMM_C_COL && b_layout != NEOGEMM_B_NK) continue;
+    if ((c.variant == NEOGEMM_VARIANT_T192x256_W4 || c.variant == NEOGEMM_VARIANT_T96x128_W4) && c_layout == NEOGEMM_C_COL &&
+        b_layout != NEOGEMM_B_NK)
+      continue;
+    // the small tiles have too little in flight to stream from HBM; 64x64 takes K-major operands only
+    if ((c.variant == NEOGEMM_VARIANT_T96x128_W4 || c.variant == NEOGEMM_VARIANT_T64x64_W4) && bytes > 32e6) continue;
+    if (c.variant == NEOGEMM_VARIANT_T64x64_W4 && b_layout != NEOGEMM_B_NK) continue;
     const double tiles = (double)ceil_div(rows, kVariants[c.variant].bm) * (double)ceil_div(cols, kVariants[c.variant].bn);
     for (int sp : kSplits) {
       if (sp > 1 && ktiles / sp < 2) break;  // at least 128 deep per split
@@ -1314,8 +1330,32 @@ static const std::vector<PlanEntry>& plan_table() {
   }();
   return table;
 }
+static void plan_uncached(int64_t M, int64_t N, int64_t K, bool aligned, int c_layout, int* variant, int* split_k,
+                          int64_t batch, int b_layout);
+// The cost model walks every (tile, split) candidate: a few microseconds on the host, as long as a small GEMM takes
+// on the GPU.  A caller in a loop repeats a handful of shapes, so each thread remembers its last few answers.
 static void plan(int64_t M, int64_t N, int64_t K, bool aligned, int c_layout, int* variant, int* split_k,
                  int64_t batch = 1, int b_layout = NEOGEMM_B_KN) {
+  struct Memo {
+    int64_t M = -1, N = -1, K = -1, batch = -1;
+    int b_layout = -1, c_layout = -1, aligned = -1, variant = 0, split_k = 0;
+  };
+  static thread_local Memo memo[32];  // the workspace query alone asks for four layouts of a shape
+  static thread_local unsigned next = 0;
+  for (const Memo& m : memo)
+    if (m.M == M && m.N == N && m.K == K && m.batch == batch && m.b_layout == b_layout && m.c_layout == c_layout &&
+        m.aligned == (int)aligned) {
+      *variant = m.variant;
+      *split_k = m.split_k;
+      return;
+    }
+  plan_uncached(M, N, K, aligned, c_layout, variant, split_k, batch, b_layout);
+  Memo& m = memo[next++ & 31];
+  m.M = M, m.N = N, m.K = K, m.batch = batch, m.b_layout = b_layout, m.c_layout = c_layout, m.aligned = (int)aligned;
+  m.variant = *variant, m.split_k = *split_k;
+}
+static void plan_uncached(int64_t M, int64_t N, int64_t K, bool aligned, int c_layout, int* variant, int* split_k,
+                          int64_t batch, int b_layout) {
   if (aligned && K > 0 && batch == 1) {
     for (const PlanEntry& e : plan_table())
       if (e.M == M && e.N == N && e.K == K && e.c_layout == c_layout && e.b_layout == b_layout) {
@@ -1423,8 +1463,7 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
       ccol = !ccol;  // a row-major C[m][n] is the column-major C^T
     }
     auto go = [&](auto kern, size_t lds) -> hipError_t {
-      static std::atomic<uint64_t> attr_done{0};  // per instantiation
-      if (hipError_t e = allow_lds(kern, lds, attr_done); e != hipSuccess) return e;
+      if (hipError_t e = allow_lds(kern, lds); e != hipSuccess) return e;
       kern<<<dim3(ceil_div(sa.N, 64)), 256, lds, st>>>(sa);
       return hipGetLastError();
     };
@@ -1509,6 +1548,8 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
     case NEOGEMM_VARIANT_T64x128_W4: e = launch_tile<64, 128, 1, 4>(a, ak, bk, st); break;
     case NEOGEMM_VARIANT_T128x128_W4S: e = launch_tile<128, 128, 1, 4>(a, ak, bk, st); break;
     case NEOGEMM_VARIANT_T192x256_W4: e = launch_tile<192, 256, 2, 2>(a, ak, bk, st); break;
+    case NEOGEMM_VARIANT_T96x128_W4: e = launch_tile<96, 128, 2, 2>(a, ak, bk, st); break;
+    case NEOGEMM_VARIANT_T64x64_W4: e = launch_tile<64, 64, 2, 2>(a, ak, bk, st); break;
     default: return NEOGEMM_ERR_BAD_ARG;
   }
   if (e != hipSuccess) {

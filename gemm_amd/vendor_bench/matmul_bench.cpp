@@ -190,6 +190,89 @@ __global__ __launch_bounds__(256) void mfma_ceiling_kernel(const cbf16x8* frags,
   out[blockIdx.x * 256 + threadIdx.x] = total;
 }
 
+// The same MFMA sequence (16x16x32) with, one by one, the other activities of a GEMM main loop at the rates of the
+// 256x256 tile kernel, none of which changes what is computed — so the drop in rate is what the activity costs at
+// the chip's power limit:
+//   PARTS & 1  operand fragments are read from LDS every pass (16 x ds_read_b128 per wave: 64 KiB per CU and pass)
+//              into a second register copy, as the kernel's double-buffered fragments are
+//   PARTS & 2  direct-to-LDS loads, 8 KiB per wave and pass (32 KiB per CU and pass: a 64-deep tile of A and of B per
+//              two passes), from a 64 KiB region per workgroup that stays in the L2
+//   PARTS & 4  a workgroup barrier per pass
+//   PARTS & 8  the matrix cores idle a fifth of the time (s_sleep after every pass): same work, lower utilisation
+template <int PARTS>
+__global__ __launch_bounds__(256) void gemm_like_kernel(const cbf16x8* frags, const char* src, float* out, int passes) {
+  extern __shared__ __attribute__((aligned(1024))) char smem[];  // 128 KiB of fragments + 32 KiB load ring
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  typedef __attribute__((address_space(3))) cbf16x8 lds_frag;
+  lds_frag* myfr = (lds_frag*)(__attribute__((address_space(3))) char*)smem + wave * 2048 + lane;  // [set][16][64 lanes]
+  cbf16x8 a[2][8], b[2][8];
+#pragma unroll
+  for (int s = 0; s < 2; ++s)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      a[s][i] = frags[((s * 2 + 0) * 8 + i) * 256 + threadIdx.x];
+      b[s][i] = frags[((s * 2 + 1) * 8 + i) * 256 + threadIdx.x];
+      myfr[(s * 16 + i) * 64] = a[s][i];
+      myfr[(s * 16 + 8 + i) * 64] = b[s][i];
+    }
+  __syncthreads();
+  const uint32_t ring = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem + 131072 + wave * 8192;
+  const uint64_t base = (uint64_t)src + (uint64_t)blockIdx.x * 65536;
+  typedef __attribute__((ext_vector_type(4))) int ci32x4;
+  const ci32x4 rsrc = {(int)(uint32_t)base, (int)(uint32_t)(base >> 32), 65536, 0x00020000};
+  const uint32_t voff = lane * 16;
+  cf32x4 acc[8][8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[i][j] = cf32x4{0.f, 0.f, 0.f, 0.f};
+  for (int p = 0; p < passes; p += 2) {
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      asm volatile("" ::: "memory");  // the LDS reads of a pass stay in that pass
+      if constexpr ((PARTS & 2) != 0) {
+        // at most the 8 loads of the pass before stay in flight
+        asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+        const uint32_t soff = (uint32_t)((wave * 16384 + ((p + s) & 1) * 8192) & 65535);
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0" ::"s"(ring) : "memory");
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          asm volatile("buffer_load_dwordx4 %0, %1, %2 offen offset:%3 sc1 lds" ::"v"(voff), "s"(rsrc), "s"(soff), "n"(j * 1024)
+                       : "memory");
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0" ::"s"(ring + 4096) : "memory");
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          asm volatile("buffer_load_dwordx4 %0, %1, %2 offen offset:%3 sc1 lds" ::"v"(voff), "s"(rsrc), "s"(soff + 4096),
+                       "n"(j * 1024)
+                       : "memory");
+      }
+#pragma unroll
+      for (int c = 0; c < 8; ++c) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+          asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[i][c]) : "v"(b[s][c]), "v"(a[s][i]));
+        if constexpr ((PARTS & 1) != 0) {
+          // two fragment reads per eight MFMAs: the other copy is refilled while this one is in use
+          a[s ^ 1][c] = myfr[((s ^ 1) * 16 + c) * 64];
+          b[s ^ 1][c] = myfr[((s ^ 1) * 16 + 8 + c) * 64];
+        }
+      }
+      if constexpr ((PARTS & 4) != 0) __builtin_amdgcn_s_barrier();
+      if constexpr ((PARTS & 8) != 0) __builtin_amdgcn_s_sleep(4);  // 256 cycles after 1024 cycles of MFMAs
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+  float total = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      asm volatile("" : "+a"(acc[i][j]));
+      total += acc[i][j][0] + acc[i][j][1] + acc[i][j][2] + acc[i][j][3];
+    }
+  out[blockIdx.x * 256 + threadIdx.x] = total;
+}
+
 static int run_ceiling(int preheat_ms) {
   hipStream_t st;
   HIP_OK(hipStreamCreate(&st));
@@ -238,6 +321,49 @@ static int run_ceiling(int preheat_ms) {
            "\"implied_mhz\": %.0f, \"workgroups\": %d, \"waves_per_simd\": 1}\n",
            c.insn, c.data, ms, tflops, tflops / 25.0, tflops * 1e12 / (256.0 * 4 * 1024.0) / 1e6, wgs);
     fflush(stdout);
+  }
+  // the MFMA sequence next to the other parts of a GEMM main loop, N(0,1) operands
+  {
+    void* dsrc;
+    const size_t src_bytes = (size_t)wgs * 65536;
+    std::vector<uint16_t> hs(src_bytes / 2);
+    for (auto& v : hs) v = f2bf(nd(rng) * sc);
+    HIP_OK(hipMalloc(&dsrc, src_bytes));
+    HIP_OK(hipMemcpy(dsrc, hs.data(), src_bytes, hipMemcpyHostToDevice));
+    const size_t lds = 131072 + 32768;
+    struct Like { int parts; const char* name; void (*kern)(const cbf16x8*, const char*, float*, int); };
+    const Like likes[] = {{0, "mfma", gemm_like_kernel<0>},
+                          {8, "mfma at 80% duty", gemm_like_kernel<8>},
+                          {1, "mfma+lds_reads", gemm_like_kernel<1>},
+                          {2, "mfma+l2_to_lds_loads", gemm_like_kernel<2>},
+                          {3, "mfma+lds_reads+l2_to_lds_loads", gemm_like_kernel<3>},
+                          {7, "mfma+lds_reads+l2_to_lds_loads+barrier", gemm_like_kernel<7>}};
+    for (int zero = 0; zero < 2; ++zero)
+    for (const Like& l : likes) {
+      // on all-zero operands the chip is not power-limited: what an activity costs there is issue slots and stalls
+      if (zero) HIP_OK(hipMemset(dsrc, 0, src_bytes));
+      const void* fr = zero ? dz : dfr;
+      HIP_OK(hipFuncSetAttribute((const void*)l.kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+      auto launch = [&](int) { l.kern<<<wgs, 256, lds, st>>>((const cbf16x8*)fr, (const char*)dsrc, (float*)dout, passes); };
+      hipEvent_t e0, e1;
+      HIP_OK(hipEventCreate(&e0));
+      HIP_OK(hipEventCreate(&e1));
+      for (float heated = 0.f; heated < (float)preheat_ms;) {
+        HIP_OK(hipEventRecord(e0, st));
+        for (int i = 0; i < 20; ++i) launch(i);
+        HIP_OK(hipEventRecord(e1, st));
+        HIP_OK(hipEventSynchronize(e1));
+        float t;
+        HIP_OK(hipEventElapsedTime(&t, e0, e1));
+        heated += t;
+      }
+      HIP_OK(hipGetLastError());
+      const double ms = time_ms(launch, 40, st);
+      const double tflops = flop / ms / 1e9;
+      printf("{\"ceiling\": \"gemm_like\", \"parts\": \"%s\", \"operands\": \"%s\", \"ms\": %.5f, \"tflops\": %.1f, "
+             "\"pct_of_2500\": %.2f}\n", l.name, zero ? "zeros" : "randn", ms, tflops, tflops / 25.0);
+      fflush(stdout);
+    }
   }
   return 0;
 }

@@ -58,7 +58,12 @@ extern "C" {
 /* 192x256, 4 wave64 (2x2): 3/4 of the 256x256 tile, for tile counts that fill the 256 CUs better (3072, 6144 ...);
    the operand that supplies the 192 rows must be K-major (A for row-major C; B [N,K] for column-major C). */
 #define NEOGEMM_VARIANT_T192x256_W4 12
-#define NEOGEMM_VARIANT_COUNT 13
+/* 96x128, 4 wave64 (2x2): three quarters of the 128x128 tile (1536 = 16 x 96: 192 workgroups where 128x128 gives 144);
+   the 96 rows must come from a K-major operand, as for 192x256. */
+#define NEOGEMM_VARIANT_T96x128_W4 13
+/* 64x64, 4 wave64 (2x2), both operands K-major (B [N,K]): small problems that would leave most CUs idle otherwise. */
+#define NEOGEMM_VARIANT_T64x64_W4 14
+#define NEOGEMM_VARIANT_COUNT 15
 
 /*
  * C = A * op(B), bf16 in, fp32 accumulate, bf16 out.

@@ -22,11 +22,35 @@ from oracle import gemm_oracle as o
 pytestmark = pytest.mark.gpu
 
 TILE_VARIANTS = [g.VARIANT_T256x256_W8, g.VARIANT_T256x256_W4, g.VARIANT_T128x128_W4, g.VARIANT_T256x128_W4,
-                 g.VARIANT_T128x256_W4, g.VARIANT_T64x128_W4, g.VARIANT_T128x128_W4S, g.VARIANT_T192x256_W4]
+                 g.VARIANT_T128x256_W4, g.VARIANT_T64x128_W4, g.VARIANT_T128x128_W4S, g.VARIANT_T192x256_W4,
+                 g.VARIANT_T96x128_W4, g.VARIANT_T64x64_W4]
 ALL_VARIANTS = [g.VARIANT_GENERIC] + TILE_VARIANTS
 
 
-def run_abi(A, B, dev, b_layout=g.B_KN, c_layout=g.C_ROW, variant=None, split_k=0, group_m=0, strict=False):
+TILE_SHAPE = {g.VARIANT_T256x256_W8: (256, 256), g.VARIANT_T256x256_W4: (256, 256), g.VARIANT_T128x128_W4: (128, 128),
+              g.VARIANT_T256x128_W4: (256, 128), g.VARIANT_T128x256_W4: (128, 256), g.VARIANT_T64x128_W4: (64, 128),
+              g.VARIANT_T128x128_W4S: (128, 128), g.VARIANT_T192x256_W4: (192, 256), g.VARIANT_T96x128_W4: (96, 128),
+              g.VARIANT_T64x64_W4: (64, 64)}
+
+
+def supported(variant, b_layout, c_layout):
+    """Whether a forced tile variant takes this pair of layouts.  The kernels write row-major output, so a
+    column-major C exchanges the operands' roles; the side of the tile that an MN-major operand (B [K,N]) lands on
+    must be a power of two of at least 128 rows.  Everything else is refused with ERR_UNSUPPORTED, never mis-run."""
+    if variant is None or variant not in TILE_SHAPE:
+        return True
+    bm, bn = TILE_SHAPE[variant]
+    ok = lambda rows: rows >= 128 and rows & (rows - 1) == 0
+    if b_layout == g.B_NK:
+        return True
+    return ok(bn) if c_layout == g.C_ROW else ok(bm)
+
+
+def cells(variants, b_layouts=(g.B_KN, g.B_NK), c_layouts=(g.C_ROW, g.C_COL)):
+    return [(v, b, c) for v in variants for b in b_layouts for c in c_layouts if supported(v, b, c)]
+
+
+def run_abi(A, B, dev, b_layout=g.B_KN, c_layout=g.C_ROW, variant=None, split_k=0, group_m=0, strict=True):
     """A [M,K] and B ([K,N] or [N,K]) are CPU bf16 tensors; returns the [M,N] result on the CPU."""
     M, K = A.shape
     N = B.shape[1] if b_layout == g.B_KN else B.shape[0]
@@ -36,12 +60,8 @@ def run_abi(A, B, dev, b_layout=g.B_KN, c_layout=g.C_ROW, variant=None, split_k=
     try:
         g.gemm_into(Ad, Bd, C, M, N, K, max(K, 1), max(N if b_layout == g.B_KN else K, 1),
                     max(N if c_layout == g.C_ROW else M, 1), b_layout, c_layout, variant, split_k, group_m)
-    except g.NeoGemmError as e:
-        if e.status == _abi.ERR_UNSUPPORTED and variant not in (None, g.VARIANT_GENERIC) and not strict:
-            # a forced tile variant may refuse a layout (an MN-major operand needs a tile >= 128 wide, ld >= tile,
-            # rows % 8 == 0): refusing is the documented behaviour, mis-running would not be
-            pytest.skip(f"variant {variant} refuses this layout/shape (status {e.status})")
-        raise
+    except g.NeoGemmError:
+        raise   # the parametrizations below only name (variant, layout) cells the library documents as supported
     torch.cuda.synchronize()
     C = C.cpu()
     return C if c_layout == g.C_ROW else C.t().contiguous()
@@ -51,12 +71,32 @@ def layouts(Bkn, b_layout):
     return Bkn if b_layout == g.B_KN else Bkn.t().contiguous()
 
 
+# the 64x64 tile takes K-major operands only (B [N,K]); tests that force a variant on one layout use this one for it
+NK_ONLY = (g.VARIANT_T64x64_W4,)
+
+
+def home_layout(variant):
+    return g.B_NK if variant in NK_ONLY else g.B_KN
+
+
 # ------------------------------------------------------------------------------------------------
 # known answers: bit-exact, every variant, every layout
 # ------------------------------------------------------------------------------------------------
-@pytest.mark.parametrize("variant", ALL_VARIANTS)
-@pytest.mark.parametrize("b_layout", [g.B_KN, g.B_NK])
-@pytest.mark.parametrize("c_layout", [g.C_ROW, g.C_COL])
+def test_unsupported_cells_are_refused(dev):
+    A = torch.zeros(256, 256, dtype=torch.bfloat16, device=dev)
+    refused = 0
+    for v in TILE_VARIANTS:
+        for b in (g.B_KN, g.B_NK):
+            for c in (g.C_ROW, g.C_COL):
+                if not supported(v, b, c):
+                    st = _abi.gemm_raw(A.data_ptr(), A.data_ptr(), A.data_ptr(), 256, 256, 256, 256, 256, 256, b, c, 0, 0, 0, v, 1, 0)
+                    assert st == _abi.ERR_UNSUPPORTED, (v, b, c, st)
+                    refused += 1
+    torch.cuda.synchronize()
+    assert refused == 5   # 64x128, 192x256, 96x128 with B [K,N] and column-major C; 64x64 with B [K,N] either way
+
+
+@pytest.mark.parametrize("variant,b_layout,c_layout", cells(ALL_VARIANTS))
 def test_identity_and_permutation(dev, variant, b_layout, c_layout):
     n = 384
     A, _ = o.make_inputs(n, n, n, seed=1)
@@ -76,11 +116,14 @@ def test_exact_small_integers(dev, variant):
     B = torch.from_numpy(rng.integers(-8, 9, size=(K, N)).astype(np.float32)).to(torch.bfloat16)
     want = (A.to(torch.int64) @ B.to(torch.int64)).float().to(torch.bfloat16)   # |sum| < 2^24: fp32 exact
     for b_layout in (g.B_KN, g.B_NK):
+        if b_layout == g.B_KN and variant in NK_ONLY:
+            continue
         got = run_abi(A, layouts(B, b_layout), dev, b_layout, g.C_ROW, variant)
         assert torch.equal(got, want)
     if variant != g.VARIANT_GENERIC:
+        bl = home_layout(variant)
         for split in (2, 3, 7):
-            assert torch.equal(run_abi(A, B, dev, variant=variant, split_k=split), want)
+            assert torch.equal(run_abi(A, layouts(B, bl), dev, bl, variant=variant, split_k=split), want)
 
 
 @pytest.mark.parametrize("K", [8, 256, 264, 1000, 4096])
@@ -120,9 +163,7 @@ def test_golden(dev, name):
 # ------------------------------------------------------------------------------------------------
 # seeded random parity at the benchmark configurations
 # ------------------------------------------------------------------------------------------------
-@pytest.mark.parametrize("variant", [None] + ALL_VARIANTS)
-@pytest.mark.parametrize("b_layout", [g.B_KN, g.B_NK])
-@pytest.mark.parametrize("c_layout", [g.C_ROW, g.C_COL])
+@pytest.mark.parametrize("variant,b_layout,c_layout", cells([None] + ALL_VARIANTS))
 def test_parity_512(dev, variant, b_layout, c_layout):
     A, Bkn = o.make_inputs(512, 512, 512, seed=0)
     got = run_abi(A, layouts(Bkn, b_layout), dev, b_layout, c_layout, variant)
@@ -175,7 +216,8 @@ def test_parity_tall_k(dev):
 def test_split_k(dev, variant, split):
     M, N, K = 200, 392, 2056
     A, Bkn = o.make_inputs(M, N, K, seed=8)
-    got = run_abi(A, Bkn, dev, variant=variant, split_k=split)
+    bl = home_layout(variant)
+    got = run_abi(A, layouts(Bkn, bl), dev, bl, variant=variant, split_k=split)
     o.assert_parity(got, A, Bkn, what=f"split {split} v{variant}")
 
 
@@ -210,9 +252,12 @@ def test_ragged_shapes_forced_tile_kernels(dev, variant, M, N, K):
 # The tile kernels stage K in 64-deep tiles / 32-deep slabs with a prologue, a steady loop that is entered
 # from seven K tiles on and unrolls two periods, and a tail: every K below walks a different way through
 # them (tile counts 1..13, with and without a partial last tile), once per operand combination.
-@pytest.mark.parametrize("variant", [g.VARIANT_T256x256_W4, g.VARIANT_T256x256_W8, g.VARIANT_T128x128_W4])
+@pytest.mark.parametrize("variant", [g.VARIANT_T256x256_W4, g.VARIANT_T256x256_W8, g.VARIANT_T128x128_W4, g.VARIANT_T96x128_W4,
+                                     g.VARIANT_T64x64_W4])
 @pytest.mark.parametrize("b_layout,c_layout", [(g.B_KN, g.C_ROW), (g.B_NK, g.C_ROW), (g.B_KN, g.C_COL)])
 def test_k_loop_transitions(dev, variant, b_layout, c_layout):
+    if not supported(variant, b_layout, c_layout):
+        b_layout = g.B_NK   # the same walk through the K loop on the layouts this tile takes
     M, N = 264, 392   # two tile rows/columns of the largest tile, ragged, both multiples of 8
     for K in (64, 72, 120, 128, 136, 192, 200, 256, 320, 384, 440, 448, 456, 512, 576, 640, 704, 768, 776, 832):
         A, Bkn = o.make_inputs(M, N, K, seed=K)
@@ -411,8 +456,9 @@ def test_variants_agree_bitwise_on_exact_data(dev):
     B = torch.from_numpy(rng.integers(-4, 5, size=(K, N)).astype(np.float32)).to(torch.bfloat16)
     base = run_abi(A, B, dev, variant=g.VARIANT_GENERIC)
     for v in TILE_VARIANTS:
+        bl = home_layout(v)
         for gm in (1, 3, 8):
-            assert torch.equal(run_abi(A, B, dev, variant=v, group_m=gm), base)
+            assert torch.equal(run_abi(A, layouts(B, bl), dev, bl, variant=v, group_m=gm), base)
 
 
 # ------------------------------------------------------------------------------------------------
