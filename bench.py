@@ -81,6 +81,10 @@ def power_ceiling(preheat_ms):
             # the 16x16x32 sequence on N(0,1) operands next to the other parts of a GEMM main loop, at the tile kernel's rates
             out.setdefault("with_gemm_parts_" + r["operands"], {})[r["parts"]] = r["tflops"]
             continue
+        if r["ceiling"] == "mfma_order":
+            # the same 128 MFMAs of a wave tile in different orders (the tile kernel uses the 2x2-block walk)
+            out.setdefault("by_mfma_order_" + r["operands"], {})[r["order"]] = r["tflops"]
+            continue
         short = "16x16x32" if "16x16x32" in r["ceiling"] else "32x32x16"
         out[f"{short}_{r['operands']}"] = r["tflops"]
         out[f"{short}_{r['operands']}_mhz"] = r["implied_mhz"]

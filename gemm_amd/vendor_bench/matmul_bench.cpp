@@ -18,6 +18,8 @@
 // operands (two register sets alternating, so that the operand buses toggle as they do on fresh data).  On
 // zeros the chip holds its top clock; on random data it is power-limited and the clock drops: that rate, not
 // the data-sheet peak, bounds any GEMM kernel on such inputs on this chip.
+// It then runs the 128 MFMAs of a wave tile in four different orders (mfma_order_kernel) and the sequence next to the
+// other activities of a GEMM main loop (gemm_like_kernel): what each costs at the power limit.
 #include <hip/hip_runtime.h>
 #include <hipblaslt/hipblaslt.h>
 #include <rocblas/rocblas.h>
@@ -29,6 +31,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <random>
+#include <utility>
 #include <vector>
 
 #include "neogemm.h"
@@ -273,6 +276,70 @@ __global__ __launch_bounds__(256) void gemm_like_kernel(const cbf16x8* frags, co
   out[blockIdx.x * 256 + threadIdx.x] = total;
 }
 
+// The order in which a wave visits its 8x8 accumulator tiles over two K steps (128 MFMAs, the same instructions on
+// the same operands every time): what changes is how many operand registers and accumulators differ from one MFMA
+// to the next, and with it the power the sequence draws.
+//   ORDER 0  column by column: the B fragment is held for eight MFMAs, the A fragment changes every time
+//   ORDER 1  2x2 blocks of tiles, the blocks in rows of alternating direction: one of the two operands is held at
+//            every step (the walk of neogemm's tile kernel)
+//   ORDER 2  along diagonals: both operands change at every step
+//   ORDER 3  the walk of ORDER 1, but both K steps of a tile back to back: every second MFMA accumulates into the
+//            tile the one before it wrote (both operands change at every step)
+template <class F, int... I>
+__device__ __forceinline__ void order_for_impl(F&& f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+constexpr int order_c(int order, int m) {  // m: 0..63, position in the walk over the tiles
+  if (order == 0) return m / 8;
+  if (order == 2) return (m / 8 + m % 8) % 8;
+  return ((m / 4) / 4) * 2 + ((m % 4) >> 1);
+}
+constexpr int order_i(int order, int m) {
+  if (order == 0 || order == 2) return m % 8;
+  const int blk = m / 4, in = m % 4, bc = blk / 4;
+  const int bi = (bc & 1) ? 3 - blk % 4 : blk % 4;
+  return bi * 2 + ((in & 1) ^ (in >> 1));
+}
+__device__ __forceinline__ void order_mfma(cf32x4& acc, cbf16x8 x, cbf16x8 y) {
+  asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(x), "v"(y));
+}
+template <int ORDER>
+__global__ __launch_bounds__(256) void mfma_order_kernel(const cbf16x8* frags, float* out, int passes) {
+  cbf16x8 a[2][8], b[2][8];
+#pragma unroll
+  for (int s = 0; s < 2; ++s)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      a[s][i] = frags[((s * 2 + 0) * 8 + i) * 256 + threadIdx.x];
+      b[s][i] = frags[((s * 2 + 1) * 8 + i) * 256 + threadIdx.x];
+    }
+  cf32x4 acc[8][8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[i][j] = cf32x4{0.f, 0.f, 0.f, 0.f};
+  for (int p = 0; p < passes; p += 2) {
+    order_for_impl(
+        [&](auto mc) {
+          constexpr int m = decltype(mc)::value;
+          constexpr int s = ORDER == 3 ? m % 2 : m / 64, t = ORDER == 3 ? m / 2 : m % 64;
+          constexpr int c = order_c(ORDER, t), i = order_i(ORDER, t);
+          order_mfma(acc[i][c], b[s][c], a[s][i]);
+        },
+        std::make_integer_sequence<int, 128>{});
+  }
+  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+  float total = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      asm volatile("" : "+a"(acc[i][j]));
+      total += acc[i][j][0] + acc[i][j][1] + acc[i][j][2] + acc[i][j][3];
+    }
+  out[blockIdx.x * 256 + threadIdx.x] = total;
+}
+
 static int run_ceiling(int preheat_ms) {
   hipStream_t st;
   HIP_OK(hipStreamCreate(&st));
@@ -321,6 +388,34 @@ static int run_ceiling(int preheat_ms) {
            "\"implied_mhz\": %.0f, \"workgroups\": %d, \"waves_per_simd\": 1}\n",
            c.insn, c.data, ms, tflops, tflops / 25.0, tflops * 1e12 / (256.0 * 4 * 1024.0) / 1e6, wgs);
     fflush(stdout);
+  }
+  // the order of the MFMAs of a wave tile, N(0,1) operands
+  {
+    struct Ord { const char* name; void (*kern)(const cbf16x8*, float*, int); };
+    const Ord ords[] = {{"column by column", mfma_order_kernel<0>}, {"2x2 blocks, serpentine", mfma_order_kernel<1>},
+                        {"diagonals (both operands change)", mfma_order_kernel<2>},
+                        {"2x2 blocks, both K steps of a tile back to back", mfma_order_kernel<3>}};
+    for (const Ord& o : ords) {
+      auto launch = [&](int) { o.kern<<<wgs, 256, 0, st>>>((const cbf16x8*)dfr, (float*)dout, passes); };
+      hipEvent_t e0, e1;
+      HIP_OK(hipEventCreate(&e0));
+      HIP_OK(hipEventCreate(&e1));
+      for (float heated = 0.f; heated < (float)preheat_ms;) {
+        HIP_OK(hipEventRecord(e0, st));
+        for (int i = 0; i < 20; ++i) launch(i);
+        HIP_OK(hipEventRecord(e1, st));
+        HIP_OK(hipEventSynchronize(e1));
+        float t;
+        HIP_OK(hipEventElapsedTime(&t, e0, e1));
+        heated += t;
+      }
+      HIP_OK(hipGetLastError());
+      const double ms = time_ms(launch, 40, st);
+      const double tflops = flop / ms / 1e9;
+      printf("{\"ceiling\": \"mfma_order\", \"order\": \"%s\", \"operands\": \"randn\", \"ms\": %.5f, \"tflops\": %.1f, "
+             "\"pct_of_2500\": %.2f}\n", o.name, ms, tflops, tflops / 25.0);
+      fflush(stdout);
+    }
   }
   // the MFMA sequence next to the other parts of a GEMM main loop, N(0,1) operands
   {
