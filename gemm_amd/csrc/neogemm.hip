@@ -30,7 +30,7 @@
 #else
 #define NEOGEMM_HAS_PART(p) 1
 #endif
-#define NEOGEMM_PARTS 8
+#define NEOGEMM_PARTS 9
 
 namespace neogemm {
 
@@ -141,6 +141,29 @@ struct TileArgs {
   int batch;
 };
 
+// Workgroup id -> (K split, output tile).  Consecutive ids land on different XCDs (round-robin over the 8
+// dies, each with its own L2), so id%8 selects a contiguous slice of the work order, and the work
+// order walks, split by split, group_m tile-rows at a time: a slice is a compact block of C for one
+// range of K (with 8 splits every XCD owns one of them and fetches its share of A and B once:
+// 1024x1024x32768 went from 70 to 62 us).
+template <int BM, int BN>
+__device__ __forceinline__ void tile_of_workgroup(const TileArgs& p, int& m0, int& n0, int& kz) {
+  const int total = p.ntm * p.ntn;
+  const int work = total * p.ksplit;
+  const int pid = blockIdx.x;
+  const int q = work >> 3, r = work & 7, x = pid & 7;
+  const int w = x * q + (x < r ? x : r) + (pid >> 3);
+  kz = w / total;
+  const int lin = w - kz * total;
+  const int per_group = p.group_m * p.ntn;
+  const int g = lin / per_group;
+  const int first = g * p.group_m;
+  const int gsz = (p.ntm - first) < p.group_m ? (p.ntm - first) : p.group_m;
+  const int rem = lin - g * per_group;
+  m0 = (first + rem % gsz) * BM;
+  n0 = (rem / gsz) * BN;
+}
+
 // Global -> LDS side of one operand: which 16 bytes each lane fetches for each of this wave's
 // 1 KiB loads of a unit (a 64-deep tile if K-major, a 32-deep slab if MN-major), and the buffer
 // resource that walks along K.
@@ -211,12 +234,14 @@ struct Operand {
     }
   }
 
-  __device__ __forceinline__ i32x4 rsrc() const {
+  // live == false: a resource of size zero, every lane out of range: the loads fill their LDS bytes with zeros and
+  // touch no memory (a unit past the end of K)
+  __device__ __forceinline__ i32x4 rsrc(bool live = true) const {
     i32x4 r;
     const uint64_t b = base - VOFF_BIAS;
     r[0] = (int)(uint32_t)b;
     r[1] = (int)(uint32_t)(b >> 32);  // a 48-bit address: bits 16.. (stride, swizzle) stay 0
-    r[2] = (int)0x80000000u;
+    r[2] = live ? (int)0x80000000u : 0;
     r[3] = 0x00020000;
     return r;
   }
@@ -300,6 +325,147 @@ __device__ __forceinline__ bf16x8 with_half(bf16x8 f, i16x4 h, int which) {
   return __builtin_bit_cast(bf16x8, r);
 }
 
+// Where the accumulator tile of a wave lies in C: local (row, column) of the wave tile -> global.  Within an aligned
+// run of 16 local rows / 8 local columns the global ones are consecutive.
+struct BlockMap {  // one block
+  int r0, c0;
+  __device__ __forceinline__ int row(int l) const { return r0 + l; }
+  __device__ __forceinline__ int col(int l) const { return c0 + l; }
+};
+struct QuadMap {  // local 64-row / 64-column halves lie 128 apart (gemm_chain_kernel)
+  int r0, c0;
+  __device__ __forceinline__ int row(int l) const { return r0 + ((l >> 6) << 7) + (l & 63); }
+  __device__ __forceinline__ int col(int l) const { return c0 + ((l >> 6) << 7) + (l & 63); }
+};
+
+// Epilogue of the tile kernels: the TM x TN accumulator tiles of a wave (NW waves per workgroup, LDS_BYTES of LDS
+// that the main loop is done with) go to C as bf16, or to the split-K partials as fp32.
+template <int TM, int TN, int NW, uint32_t LDS_BYTES, class Map>
+__device__ __forceinline__ void store_wave_tile(f32x4 (&acc)[TM][TN], const TileArgs& p, char* gC, int kz, int lane,
+                                                int wave, uint32_t lds0, const Map map) {
+  constexpr int WTM = TM * 16, WTN = TN * 16;
+  // Epilogue: lane holds, per 16x16 tile, output row (lane & 15) and 4 consecutive columns 4*(lane >> 4)..+3.
+  const int row_l = lane & 15, colq = (lane >> 4) * 4;
+  // An accumulator element is read out of its AGPR where it is used: left to itself the compiler copies
+  // all 256 accumulators to VGPRs ahead of the three epilogue variants below, and spills.
+  auto acc_get = [](float a) -> float {
+    float v;
+    asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(a));
+    return v;
+  };
+  // Coalesced path: the wave parks its bf16 tile in LDS (the slab ring is dead by now) and reads it back
+  // row-wise, so that a store instruction writes whole rows of the wave tile, 16 bytes per lane, instead of
+  // sixteen 32-byte pieces.  The staging tile is WTM x WTN bf16, 16-byte chunks XOR-ed with the row number
+  // so that neither the 8-byte writes (16 rows per instruction) nor the 16-byte reads collide on banks.
+  constexpr int CH = WTN / 8;        // 16-byte chunks per staged row
+  constexpr int RPI = 64 / CH;       // rows one store instruction covers
+  constexpr bool CAN_STAGE = (size_t)NW * WTM * WTN * 2 <= (size_t)LDS_BYTES && CH >= 4 && CH <= 64;
+  const bool stage = CAN_STAGE && p.ksplit == 1 && p.beta == 0.f && (((uintptr_t)gC | (uintptr_t)(p.ldc * 2)) & 15) == 0;
+  if (stage) {
+    if constexpr (CAN_STAGE) {
+      // every wave is done with the slab images (its LDS reads have returned: the MFMAs that used them
+      // were issued; wait anyway) before any wave overwrites them; so are its direct-to-LDS loads (when K is
+      // short the prologue's fully masked zero fills of later images may still be in flight)
+      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+      const uint32_t region = lds0 + (uint32_t)wave * (WTM * WTN * 2);
+      auto park = [&](auto scaled) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+          const uint32_t row = i * 16 + row_l;
+#pragma unroll
+          for (int j = 0; j < TN; ++j) {
+            bf16x4 o;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              float v = acc_get(acc[i][j][r]);
+              if constexpr (decltype(scaled)::value) v *= p.alpha;
+              o[r] = (__bf16)v;
+            }
+            const uint32_t c = 2 * j + (lane >> 5);
+            const uint32_t addr = region + row * (WTN * 2) + ((c ^ (row & (CH - 1))) << 4) + (((lane >> 4) & 1) << 3);
+            *((NEOGEMM_AS3 bf16x4*)(uintptr_t)addr) = o;
+          }
+        }
+      };
+      if (p.alpha == 1.f) park(std::false_type{});
+      else park(std::true_type{});
+      // same wave wrote and reads: LDS operations of a wave complete in order; the compiler orders them
+      const int colc = lane % CH;
+      const int col = map.col(colc * 8);
+#pragma unroll
+      for (int st = 0; st < WTM / RPI; ++st) {
+        const uint32_t row = st * RPI + lane / CH;
+        const uint32_t addr = region + row * (WTN * 2) + (((uint32_t)colc ^ (row & (CH - 1))) << 4);
+        const bf16x8 v = *((NEOGEMM_AS3 bf16x8*)(uintptr_t)addr);
+        const int grow = map.row((int)row);
+        if (grow < p.M) {
+          char* dst = gC + ((size_t)grow * p.ldc + col) * 2;
+          if (col + 7 < p.N) {
+            // C is written once and not read again here: streaming stores leave the L2 to A and B
+            __builtin_nontemporal_store(v, (bf16x8*)dst);
+          } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+              if (col + e < p.N) ((__bf16*)dst)[e] = v[e];
+          }
+        }
+      }
+    }
+  } else if (p.ksplit == 1) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int row = map.row(i * 16 + row_l);
+      if (row >= p.M) continue;
+      char* crow = gC + (size_t)row * p.ldc * 2;
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int col = map.col(j * 16 + colq);
+        f32x4 v;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) v[r] = acc_get(acc[i][j][r]) * p.alpha;
+        if (p.beta != 0.f) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            if (col + r < p.N) v[r] = __builtin_fmaf(p.beta, (float)*(const __bf16*)(crow + (size_t)(col + r) * 2), v[r]);
+        }
+        const bf16x4 o = {(__bf16)v[0], (__bf16)v[1], (__bf16)v[2], (__bf16)v[3]};
+        if (col + 3 < p.N) {
+          __builtin_nontemporal_store(o, (bf16x4*)(crow + (size_t)col * 2));
+        } else {
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            if (col + r < p.N) *(__bf16*)(crow + (size_t)(col + r) * 2) = o[r];
+        }
+      }
+    }
+  } else {
+    float* wsz = p.ws + ((size_t)blockIdx.z * p.ksplit + kz) * p.M * p.N;
+    const bool vec = (p.N & 3) == 0;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int row = map.row(i * 16 + row_l);
+      if (row >= p.M) continue;
+      float* wrow = wsz + (size_t)row * p.N;
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int col = map.col(j * 16 + colq);
+        f32x4 o;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o[r] = acc_get(acc[i][j][r]);
+        if (vec && col + 3 < p.N) {
+          *(f32x4*)(wrow + col) = o;
+        } else {
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            if (col + r < p.N) wrow[col + r] = o[r];
+        }
+      }
+    }
+  }
+}
+
 // PROF adds s_memtime stamps around the two waits of the main loop and writes, per wave,
 // {total, waiting for own loads, waiting at the barrier, epilogue} shader-clock cycles to p.prof — the
 // per-phase cycle buffer idea of the reference's harness (cublass/matmul.cu:99-106,149-165).
@@ -329,28 +495,8 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WGN, wn = wave % WGN;
 
-  // Workgroup id -> (K split, output tile).  Consecutive ids land on different XCDs (round-robin over the 8
-  // dies, each with its own L2), so id%8 selects a contiguous slice of the work order, and the work
-  // order walks, split by split, group_m tile-rows at a time: a slice is a compact block of C for one
-  // range of K (with 8 splits every XCD owns one of them and fetches its share of A and B once:
-  // 1024x1024x32768 went from 70 to 62 us).
   int m0, n0, kz;
-  {
-    const int total = p.ntm * p.ntn;
-    const int work = total * p.ksplit;
-    const int pid = blockIdx.x;
-    const int q = work >> 3, r = work & 7, x = pid & 7;
-    const int w = x * q + (x < r ? x : r) + (pid >> 3);
-    kz = w / total;
-    const int lin = w - kz * total;
-    const int per_group = p.group_m * p.ntn;
-    const int g = lin / per_group;
-    const int first = g * p.group_m;
-    const int gsz = (p.ntm - first) < p.group_m ? (p.ntm - first) : p.group_m;
-    const int rem = lin - g * per_group;
-    m0 = (first + rem % gsz) * BM;
-    n0 = (rem / gsz) * BN;
-  }
+  tile_of_workgroup<BM, BN>(p, m0, n0, kz);
   const int k_begin = kz * p.ktiles_per_split * KTILE;
   int k_end = k_begin + p.ktiles_per_split * KTILE;
   if (k_end > p.K) k_end = p.K;
@@ -656,126 +802,7 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
   unsigned long long t_main = 0;
   if constexpr (PROF) t_main = __builtin_readcyclecounter();
 
-  // Epilogue: lane holds, per 16x16 tile, output row (lane & 15) and 4 consecutive columns 4*(lane >> 4)..+3.
-  const int row_l = lane & 15, colq = (lane >> 4) * 4;
-  // An accumulator element is read out of its AGPR where it is used: left to itself the compiler copies
-  // all 256 accumulators to VGPRs ahead of the three epilogue variants below, and spills.
-  auto acc_get = [](float a) -> float {
-    float v;
-    asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(a));
-    return v;
-  };
-  // Coalesced path: the wave parks its bf16 tile in LDS (the slab ring is dead by now) and reads it back
-  // row-wise, so that a store instruction writes whole rows of the wave tile, 16 bytes per lane, instead of
-  // sixteen 32-byte pieces.  The staging tile is WTM x WTN bf16, 16-byte chunks XOR-ed with the row number
-  // so that neither the 8-byte writes (16 rows per instruction) nor the 16-byte reads collide on banks.
-  constexpr int CH = WTN / 8;        // 16-byte chunks per staged row
-  constexpr int RPI = 64 / CH;       // rows one store instruction covers
-  constexpr bool CAN_STAGE = (size_t)BM * BN * 2 <= (size_t)LDS_BYTES && CH >= 4 && CH <= 64;
-  const bool stage = CAN_STAGE && p.ksplit == 1 && p.beta == 0.f && (((uintptr_t)gC | (uintptr_t)(p.ldc * 2)) & 15) == 0;
-  if (stage) {
-    if constexpr (CAN_STAGE) {
-      // every wave is done with the slab images (its LDS reads have returned: the MFMAs that used them
-      // were issued; wait anyway) before any wave overwrites them; so are its direct-to-LDS loads (when K is
-      // short the prologue's fully masked zero fills of later images may still be in flight)
-      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-      __builtin_amdgcn_s_barrier();
-      asm volatile("" ::: "memory");
-      const uint32_t region = lds0 + (uint32_t)wave * (WTM * WTN * 2);
-      auto park = [&](auto scaled) {
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-          const uint32_t row = i * 16 + row_l;
-#pragma unroll
-          for (int j = 0; j < TN; ++j) {
-            bf16x4 o;
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-              float v = acc_get(acc[i][j][r]);
-              if constexpr (decltype(scaled)::value) v *= p.alpha;
-              o[r] = (__bf16)v;
-            }
-            const uint32_t c = 2 * j + (lane >> 5);
-            const uint32_t addr = region + row * (WTN * 2) + ((c ^ (row & (CH - 1))) << 4) + (((lane >> 4) & 1) << 3);
-            *((NEOGEMM_AS3 bf16x4*)(uintptr_t)addr) = o;
-          }
-        }
-      };
-      if (p.alpha == 1.f) park(std::false_type{});
-      else park(std::true_type{});
-      // same wave wrote and reads: LDS operations of a wave complete in order; the compiler orders them
-      const int colc = lane % CH;
-      const int col = n0 + wn * WTN + colc * 8;
-#pragma unroll
-      for (int st = 0; st < WTM / RPI; ++st) {
-        const uint32_t row = st * RPI + lane / CH;
-        const uint32_t addr = region + row * (WTN * 2) + (((uint32_t)colc ^ (row & (CH - 1))) << 4);
-        const bf16x8 v = *((NEOGEMM_AS3 bf16x8*)(uintptr_t)addr);
-        const int grow = m0 + wm * WTM + (int)row;
-        if (grow < p.M) {
-          char* dst = gC + ((size_t)grow * p.ldc + col) * 2;
-          if (col + 7 < p.N) {
-            // C is written once and not read again here: streaming stores leave the L2 to A and B
-            __builtin_nontemporal_store(v, (bf16x8*)dst);
-          } else {
-#pragma unroll
-            for (int e = 0; e < 8; ++e)
-              if (col + e < p.N) ((__bf16*)dst)[e] = v[e];
-          }
-        }
-      }
-    }
-  } else if (p.ksplit == 1) {
-#pragma unroll
-    for (int i = 0; i < TM; ++i) {
-      const int row = m0 + wm * WTM + i * 16 + row_l;
-      if (row >= p.M) continue;
-      char* crow = gC + (size_t)row * p.ldc * 2;
-#pragma unroll
-      for (int j = 0; j < TN; ++j) {
-        const int col = n0 + wn * WTN + j * 16 + colq;
-        f32x4 v;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) v[r] = acc_get(acc[i][j][r]) * p.alpha;
-        if (p.beta != 0.f) {
-#pragma unroll
-          for (int r = 0; r < 4; ++r)
-            if (col + r < p.N) v[r] = __builtin_fmaf(p.beta, (float)*(const __bf16*)(crow + (size_t)(col + r) * 2), v[r]);
-        }
-        const bf16x4 o = {(__bf16)v[0], (__bf16)v[1], (__bf16)v[2], (__bf16)v[3]};
-        if (col + 3 < p.N) {
-          __builtin_nontemporal_store(o, (bf16x4*)(crow + (size_t)col * 2));
-        } else {
-#pragma unroll
-          for (int r = 0; r < 4; ++r)
-            if (col + r < p.N) *(__bf16*)(crow + (size_t)(col + r) * 2) = o[r];
-        }
-      }
-    }
-  } else {
-    float* wsz = p.ws + ((size_t)blockIdx.z * p.ksplit + kz) * p.M * p.N;
-    const bool vec = (p.N & 3) == 0;
-#pragma unroll
-    for (int i = 0; i < TM; ++i) {
-      const int row = m0 + wm * WTM + i * 16 + row_l;
-      if (row >= p.M) continue;
-      float* wrow = wsz + (size_t)row * p.N;
-#pragma unroll
-      for (int j = 0; j < TN; ++j) {
-        const int col = n0 + wn * WTN + j * 16 + colq;
-        f32x4 o;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) o[r] = acc_get(acc[i][j][r]);
-        if (vec && col + 3 < p.N) {
-          *(f32x4*)(wrow + col) = o;
-        } else {
-#pragma unroll
-          for (int r = 0; r < 4; ++r)
-            if (col + r < p.N) wrow[col + r] = o[r];
-        }
-      }
-    }
-  }
+  store_wave_tile<TM, TN, NW, LDS_BYTES>(acc, p, gC, kz, lane, wave, lds0, BlockMap{m0 + wm * WTM, n0 + wn * WTN});
   if constexpr (PROF) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     const unsigned long long t_end = __builtin_readcyclecounter();
@@ -844,6 +871,215 @@ hipError_t launch_tile(const TileArgs& a, bool ak, bool bk, hipStream_t st) {
   }
   return hipErrorInvalidValue;
 }
+
+// ---------------------------------------------------------------------------------------------
+// 256x256 tile, K in periods of 64 (two MFMA steps), both steps of an accumulator tile back to back.
+// A v_mfma that accumulates into the tile the instruction before it wrote takes that operand from the pipeline
+// instead of the register file, and with the walk below every MFMA either does that or shares one operand
+// register with the one before it: the matrix cores alone sustain 3 % more on N(0,1) operands than with the walk
+// of gemm_tile_kernel (matmul_bench ceiling, rows mfma_order), and under the chip's power limit that is clock.
+// Both steps of a tile in a row need the fragments of two K steps in registers at once, so the roles of the operands
+// are uneven: A's sixteen fragments (8 row tiles x 2 steps) of the current period sit in registers, double-buffered
+// across periods; B streams: the wave goes through its eight column tiles in pairs, four fragments per pair, read
+// from LDS while the pair before it is being worked on.  40 fragments live at most.
+//     period q:  column pair 0..3 (32 MFMAs each): row blocks of two tiles, in alternating direction;
+//                a block (2 columns x 2 rows x 2 steps) goes (c0,i0,k0) (c0,i0,k1) (c0,i1,k0) (c0,i1,k1) (c1,i1,k0) ...
+// LDS: A two 64-deep tile images (32 KiB each), B three (K-major: a tile image; MN-major: two 32-deep slab images),
+// laid out and swizzled as in gemm_tile_kernel.  During period q a wave loads A tile q+2 over tile q (whose fragments
+// it read during the second half of period q-1) and B tile q+2 over tile q-1: all sixteen loads in the first half.
+// Two barriers per period: at its start (everyone is done reading what the period's loads overwrite) and in the
+// middle (A tile q+1 and B tile q+1, requested during period q-1, have landed: they are read during the second half).
+// K is a multiple of 128 and not split; a tile past the end of K is requested all the same, as a zero fill.
+// ---------------------------------------------------------------------------------------------
+template <bool BK>
+__global__ __launch_bounds__(256) void gemm_chain_kernel(TileArgs p) {
+  constexpr int BM = 256, BN = 256, NW = 4, TM = 8, TN = 8;
+  using OpA = Operand<BM, true, NW, 2>;
+  using OpB = Operand<BN, BK, NW, BK ? 3 : 6>;
+  constexpr uint32_t A_BYTES = 2 * 32768, B_IMG = 32768, LDS_BYTES = A_BYTES + 3 * B_IMG;
+  constexpr int IA = OpA::IPW, IB = OpB::IPW;          // loads of this wave per unit (A: a tile; B: a tile or a slab)
+  constexpr int UB = KTILE / OpB::UNIT_K, LB = IB * UB;  // B units, B loads per period
+  static_assert(IA == 8 && LB == 8, "eight loads per operand, wave and period");
+#ifndef PAIR_LANDED_AT
+#define PAIR_LANDED_AT 88
+#endif
+#ifndef PAIR_LOAD_STEP
+#define PAIR_LOAD_STEP 7
+#endif
+  constexpr int LOAD_STEP = PAIR_LOAD_STEP;  // a load behind every LOAD_STEP-th MFMA from the third on
+  constexpr int LANDED_AT = PAIR_LANDED_AT;  // MFMA of the period before which the barrier for tile q+1 sits (even, 64..96)
+
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(NEOGEMM_AS3 char*)smem;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+
+  int m0, n0, kz;
+  tile_of_workgroup<BM, BN>(p, m0, n0, kz);
+  const int klen = p.K;  // not split
+  const int ntile = klen / KTILE;
+
+  const char* gA = p.A + (size_t)blockIdx.z * p.bsa * 2;
+  const char* gB = p.B + (size_t)blockIdx.z * p.bsb * 2;
+  char* gC = p.C + (size_t)blockIdx.z * p.bsc * 2;
+  OpA opa;
+  OpB opb;
+  opa.init(gA, p.lda, p.M, m0, 0, wave, lane);
+  opb.init(gB, p.ldb, p.N, n0, 0, wave, lane);
+  FragReader<BM, true, TM> fra;
+  FragReader<BN, BK, TN> frb;
+  fra.init(lds0, wm * 128, lane);
+  frb.init(lds0 + A_BYTES, wn * 128, lane);
+
+  f32x4 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) acc[i][j][v] = 0.f;
+
+  // load l (0..7) of the tile an operand loads next, into the image at `img` (offset within the operand's region)
+  int ta = 0, tb = 0;  // tile the next A / B loads belong to
+  auto load_a = [&](auto lc, uint32_t img) {
+    constexpr int J = decltype(lc)::value;
+    if constexpr (J % 4 == 0) dma_set_m0(lds0 + img + opa.lds_w + (J / 4) * 4096);
+    opa.template issue_one<J>(opa.rsrc(ta < ntile));
+    if constexpr (J == IA - 1) {
+      opa.advance();
+      ++ta;
+    }
+  };
+  auto load_b = [&](auto lc, uint32_t img) {
+    constexpr int l = decltype(lc)::value, u = l / IB, J = l % IB;
+    if constexpr (J % 4 == 0) dma_set_m0(lds0 + A_BYTES + img + u * OpB::IMG + opb.lds_w + (J / 4) * 4096);
+    opb.template issue_one<J>(opb.rsrc(tb < ntile));
+    if constexpr (J == IB - 1) {
+      opb.advance();
+      if constexpr (u == UB - 1) ++tb;
+    }
+  };
+
+  // B fragments of column tile c (0..7), step k, from the B image at region offset `img`
+  auto read_b = [&](uint32_t img, int c, int k) -> bf16x8 {
+    if constexpr (BK) {
+      return lds_read_b128(frb.lane_off[k] + img + (uint32_t)c * 2048);
+    } else {
+      const uint32_t a = frb.lane_off[c] + img + (uint32_t)k * OpB::IMG;
+      const i16x8 v = __builtin_shufflevector(lds_read_tr16(a), lds_read_tr16(a + 4 * FragReader<BN, BK, TN>::ROWB), 0, 1, 2,
+                                              3, 4, 5, 6, 7);
+      return __builtin_bit_cast(bf16x8, v);
+    }
+  };
+
+  auto barrier = [&](auto keep, auto lgk) {
+    constexpr int KEEP = decltype(keep)::value;
+    constexpr bool LGK = decltype(lgk)::value;
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (KEEP >= 0 && LGK) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(KEEP) : "memory");
+    else if constexpr (KEEP >= 0) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(KEEP) : "memory");
+    else if constexpr (LGK) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  using NoVm = std::integral_constant<int, -1>;
+  using T = std::true_type;
+  using F = std::false_type;
+
+  // fragments: fa[buffer][row tile][step], the buffer is the tile's parity; fb[column pair parity][column][step]
+  bf16x8 fa[2][TM][2] = {}, fb[2][2][2] = {};
+
+  // prologue: tiles 0 and 1 of both operands; tile 0 of A and the first column pair of B's tile 0 into registers
+  uint32_t b_cur = 0, b_nxt = B_IMG, b_ld = 2 * B_IMG;  // B images: this period's tile, the next one's, the one being loaded
+  static_for<IA>([&](auto lc) { load_a(lc, 0); });
+  static_for<LB>([&](auto lc) { load_b(lc, b_cur); });
+  static_for<IA>([&](auto lc) { load_a(lc, 32768); });
+  static_for<LB>([&](auto lc) { load_b(lc, b_nxt); });
+  barrier(std::integral_constant<int, IA + LB>{}, F{});
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int k = 0; k < 2; ++k) fa[0][i][k] = fra.read(0, i, k);
+#pragma unroll
+  for (int c = 0; c < 2; ++c)
+#pragma unroll
+    for (int k = 0; k < 2; ++k) fb[0][c][k] = read_b(b_cur, c, k);
+
+  for (int q = 0; q < ntile; q += 2) {
+    static_for<256>([&](auto mc) {
+      constexpr int m2 = decltype(mc)::value, par = m2 / 128, m = m2 % 128;  // par: parity of the tile = A buffer and image
+      constexpr int cp = m / 32, e = m % 8;
+      constexpr int rb = (cp & 1) ? 3 - (m % 32) / 8 : (m % 32) / 8;
+      constexpr int c = e / 4, i = rb * 2 + (((e + 2) >> 2) & 1), k = e & 1;  // k ascending on every tile: the sum's order is that of gemm_tile_kernel
+      // ---- barriers
+      if constexpr (m == 0) barrier(NoVm{}, T{});                                          // the images this period loads into are free
+      if constexpr (m == LANDED_AT) barrier(std::integral_constant<int, (LANDED_AT - 2 + LOAD_STEP - 1) / LOAD_STEP < IA + LB ? (LANDED_AT - 2 + LOAD_STEP - 1) / LOAD_STEP : IA + LB>{}, F{});  // tile q+1 of A and of B has landed
+      // ---- the MFMA
+      mfma_16x16x32(acc[i][cp * 2 + c], fb[cp & 1][c][k], fa[par][i][k]);
+      // ---- LDS reads behind it
+      // B: the next column pair's four fragments, early in this one (the last pair reads the first of the next tile,
+      // which the barrier before has seen land); a K-major fragment is one 16-byte read, an MN-major one two
+      // transposing 8-byte reads, each behind an MFMA of its own
+      if constexpr (BK) {
+        if constexpr (m % 32 < 16 && (m % 4) == 1) {
+          constexpr int j = (m % 32) / 4, cc = j / 2, kk = j % 2;
+          if constexpr (cp < 3) fb[(cp + 1) & 1][cc][kk] = read_b(b_cur, (cp + 1) * 2 + cc, kk);
+          else fb[0][cc][kk] = read_b(b_nxt, cc, kk);
+        }
+      } else {
+        if constexpr (m % 32 < 16 && (m % 2) == 1) {
+          constexpr int idx = (m % 32) / 2, j = idx / 2, h = idx % 2, cc = j / 2, kk = j % 2;
+          constexpr int nb = cp < 3 ? (cp + 1) & 1 : 0, ct = cp < 3 ? (cp + 1) * 2 + cc : cc;
+          const uint32_t a = frb.lane_off[ct] + (cp < 3 ? b_cur : b_nxt) + (uint32_t)kk * OpB::IMG + h * 4 * FragReader<BN, BK, TN>::ROWB;
+          fb[nb][cc][kk] = with_half(fb[nb][cc][kk], lds_read_tr16(a), h);
+        }
+      }
+      // A: the next tile's sixteen fragments behind the even MFMAs 64..94 (B's reads sit behind odd ones); done well
+      // before the period ends, where the next one's first barrier waits for them
+      if constexpr (m >= LANDED_AT && m < LANDED_AT + 32 && (m % 2) == 0) {
+        constexpr int j = (m - LANDED_AT) / 2, ii = j / 2, kk = j % 2;
+        fa[par ^ 1][ii][kk] = fra.read((par ^ 1) * 32768, ii, kk);
+      }
+      // ---- loads behind it: all sixteen in the first half, A's tile q+2 over tile q, B's over tile q-1
+      if constexpr (m >= 2 && (m - 2) % LOAD_STEP == 0 && (m - 2) / LOAD_STEP < IA + LB) {
+        constexpr int l = (m - 2) / LOAD_STEP;
+        if constexpr (l < IA) load_a(std::integral_constant<int, l>{}, par * 32768);
+        else load_b(std::integral_constant<int, l - IA>{}, b_ld);
+      }
+      // ---- end of the period: the B images change roles
+      if constexpr (m == 127) {
+        const uint32_t t = b_cur;
+        b_cur = b_nxt;
+        b_nxt = b_ld;
+        b_ld = t;
+      }
+    });
+  }
+
+  // the last MFMAs must have left the pipe before their accumulators are read (see gemm_tile_kernel)
+  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int jn = 0; jn < TN; ++jn) asm volatile("" : "+a"(acc[i][jn]));
+  store_wave_tile<TM, TN, NW, LDS_BYTES>(acc, p, gC, kz, lane, wave, lds0, BlockMap{m0 + wm * 128, n0 + wn * 128});
+}
+
+hipError_t launch_chain(const TileArgs& a, bool bk, hipStream_t st);
+#if NEOGEMM_HAS_PART(8)
+hipError_t launch_chain(const TileArgs& a, bool bk, hipStream_t st) {
+  const size_t lds = 5 * 32768;
+  dim3 grid(a.ntm * a.ntn, 1, a.batch), block(256);
+  auto go = [&](auto kern) -> hipError_t {
+    if (hipError_t e = allow_lds(kern, lds); e != hipSuccess) return e;
+    kern<<<grid, block, lds, st>>>(a);
+    return hipGetLastError();
+  };
+  return bk ? go(gemm_chain_kernel<true>) : go(gemm_chain_kernel<false>);
+}
+#endif
 
 // The tile kernels are instantiated through launch_tile.  In a split build each part instantiates its share and
 // the others only declare it.
@@ -1197,7 +1433,7 @@ struct VariantInfo {
 };
 static const VariantInfo kVariants[NEOGEMM_VARIANT_COUNT] = {
     {0, 0, 0}, {16, 16, 4}, {256, 256, 8}, {256, 256, 4}, {128, 128, 4}, {256, 128, 4}, {128, 256, 4}, {64, 128, 4}, {128, 128, 4},
-    {16, 64, 4}, {32, 64, 4}, {64, 64, 4}, {192, 256, 4}, {96, 128, 4}, {64, 64, 4},
+    {16, 64, 4}, {32, 64, 4}, {64, 64, 4}, {192, 256, 4}, {96, 128, 4}, {64, 64, 4}, {256, 256, 4},
 };
 
 static bool is_aligned(const void* A, const void* B, const void* C, int64_t K, int64_t lda, int64_t ldb,
@@ -1299,6 +1535,11 @@ static void plan_model(int64_t M, int64_t N, int64_t K, bool aligned, int c_layo
       bs = 1;
     }
   }
+  // the 256x256 tile unsplit, K in whole periods of 128, rows from a K-major operand: the kernel that accumulates twice
+  // in a row into each tile does the same work on less power (8192^3 +1.3 %, 4096^3 +1.2 %, bit-identical results)
+  if (bv == NEOGEMM_VARIANT_T256x256_W4 && bs == 1 && K % (2 * KTILE) == 0 &&
+      (c_layout == NEOGEMM_C_ROW || b_layout == NEOGEMM_B_NK))
+    bv = NEOGEMM_VARIANT_C256x256_W4;
   *variant = bv;
   *split_k = bs;
 }
@@ -1526,7 +1767,9 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
   // of two, for its swizzle and a row count that is a multiple of 8 (16-byte chunks must not straddle the
   // matrix edge).
   auto mn_ok = [](int tile, int rows) { return tile >= 128 && (tile & (tile - 1)) == 0 && (rows & 7) == 0; };
-  const bool fits = (ak || mn_ok(vi.bm, a.M)) && (bk || mn_ok(vi.bn, a.N));
+  // (the chained 256x256 kernel takes its rows from a K-major operand only, K in whole periods of 128 and no split)
+  const bool fits = (ak || mn_ok(vi.bm, a.M)) && (bk || mn_ok(vi.bn, a.N)) &&
+                    (v != NEOGEMM_VARIANT_C256x256_W4 || (ak && K % (2 * KTILE) == 0 && s <= 1));
   if (!fits) {
     if (variant != NEOGEMM_VARIANT_AUTO) return NEOGEMM_ERR_UNSUPPORTED;
     // the planned tile is too wide for an MN-major operand: the 128x128 tile needs the least, then generic
@@ -1550,7 +1793,8 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
   a.prof = prof;
   a.alpha = alpha;
   a.beta = beta;
-  if (prof && (bt.count > 1 || a.ksplit > 1 || vi.bm != 256 || vi.bn != 256 || !ak)) return NEOGEMM_ERR_UNSUPPORTED;
+  if (prof && (bt.count > 1 || a.ksplit > 1 || vi.bm != 256 || vi.bn != 256 || !ak || v == NEOGEMM_VARIANT_C256x256_W4))
+    return NEOGEMM_ERR_UNSUPPORTED;
   if (a.ksplit > 1) {
     const size_t need = (size_t)a.ksplit * (size_t)M * (size_t)N * sizeof(float) * (size_t)bt.count;
     if (!workspace || workspace_bytes < need) return NEOGEMM_ERR_WORKSPACE;
@@ -1570,6 +1814,7 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
     case NEOGEMM_VARIANT_T192x256_W4: e = launch_tile<192, 256, 2, 2>(a, ak, bk, st); break;
     case NEOGEMM_VARIANT_T96x128_W4: e = launch_tile<96, 128, 2, 2>(a, ak, bk, st); break;
     case NEOGEMM_VARIANT_T64x64_W4: e = launch_tile<64, 64, 2, 2>(a, ak, bk, st); break;
+    case NEOGEMM_VARIANT_C256x256_W4: e = launch_chain(a, bk, st); break;
     default: return NEOGEMM_ERR_BAD_ARG;
   }
   if (e != hipSuccess) {

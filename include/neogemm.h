@@ -63,7 +63,11 @@ extern "C" {
 #define NEOGEMM_VARIANT_T96x128_W4 13
 /* 64x64, 4 wave64 (2x2), both operands K-major (B [N,K]): small problems that would leave most CUs idle otherwise. */
 #define NEOGEMM_VARIANT_T64x64_W4 14
-#define NEOGEMM_VARIANT_COUNT 15
+/* 256x256, 4 wave64 (2x2), K in periods of 64 with both MFMA steps of an accumulator tile back to back (less
+   register-file traffic per flop: what the chip's power limit rewards); the operand that supplies the rows must be
+   K-major, K a multiple of 128, no split-K. */
+#define NEOGEMM_VARIANT_C256x256_W4 15
+#define NEOGEMM_VARIANT_COUNT 16
 
 /*
  * C = A * op(B), bf16 in, fp32 accumulate, bf16 out.

@@ -22,7 +22,7 @@ HIPCC_FLAGS = [
     # packed-fp32 VALU forms are kept off for every HIP file of this project
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
-KERNEL_PARTS = 8  # NEOGEMM_PARTS in gemm_amd/csrc/neogemm.hip
+KERNEL_PARTS = 9  # NEOGEMM_PARTS in gemm_amd/csrc/neogemm.hip
 
 
 def build_kernels():

@@ -53,7 +53,11 @@ def test_plan_for_the_benchmark_configs():
     # square compute-bound shapes run a 256x256 tile kernel without split-K
     for n in (4096, 8192):
         v, s = _abi.plan(n, n, n)
-        assert v in (_abi.VARIANT_T256x256_W4, _abi.VARIANT_T256x256_W8) and s == 1
+        assert v == _abi.VARIANT_C256x256_W4 and s == 1   # K in whole periods of 128, A K-major: the chained kernel
+        assert _abi.plan(n, n, n, _abi.B_NK, _abi.C_COL) == (_abi.VARIANT_C256x256_W4, 1)   # the reference's call
+        # B [K,N] with a column-major C puts the MN-major operand on the rows, K = 8256 is not whole periods: slab kernel
+        assert _abi.plan(n, n, n, _abi.B_KN, _abi.C_COL)[0] in (_abi.VARIANT_T256x256_W4, _abi.VARIANT_T256x256_W8)
+        assert _abi.plan(n, n, n + 64)[0] in (_abi.VARIANT_T256x256_W4, _abi.VARIANT_T256x256_W8)
     # shapes with few output tiles split K and need a workspace of split * M * N floats (skinny M with a row-major C
     # runs the streaming kernel instead, without split-K)
     for M, N, K in ((16, 14336, 4096), (64, 14336, 4096), (128, 14336, 4096), (1024, 1024, 32768), (512, 512, 512)):

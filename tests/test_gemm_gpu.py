@@ -449,6 +449,63 @@ def test_properties_full_size(dev):
     assert float((lhs - rhs).abs().max()) <= tol * math.sqrt(M)
 
 
+# The chained 256x256 kernel (two MFMA steps per accumulator tile back to back, A's fragments resident, B's streamed)
+# takes K in whole periods of 128, no split-K, and its rows from a K-major operand; on those problems it must give
+# what the slab kernel gives, bit for bit (same sums in the same order).
+CHAIN_CELLS = [(g.B_KN, g.C_ROW), (g.B_NK, g.C_ROW), (g.B_NK, g.C_COL)]
+
+
+@pytest.mark.parametrize("b_layout,c_layout", CHAIN_CELLS)
+def test_chain_kernel_known_answers(dev, b_layout, c_layout):
+    v = g.VARIANT_C256x256_W4
+    n = 384
+    A, _ = o.make_inputs(n, n, n, seed=1)
+    I = torch.eye(n, dtype=torch.bfloat16)
+    assert torch.equal(run_abi(A, layouts(I, b_layout), dev, b_layout, c_layout, v), A)
+    perm = torch.randperm(n, generator=torch.Generator().manual_seed(2))
+    P = torch.zeros(n, n, dtype=torch.bfloat16)
+    P[torch.arange(n), perm] = 1
+    assert torch.equal(run_abi(P, layouts(A, b_layout), dev, b_layout, c_layout, v), A[perm])
+    rng = np.random.default_rng(11)
+    M, N, K = 264, 328, 256   # ragged in M and N
+    Ai = torch.from_numpy(rng.integers(-8, 9, size=(M, K)).astype(np.float32)).to(torch.bfloat16)
+    Bi = torch.from_numpy(rng.integers(-8, 9, size=(K, N)).astype(np.float32)).to(torch.bfloat16)
+    want = (Ai.to(torch.int64) @ Bi.to(torch.int64)).float().to(torch.bfloat16)
+    for gm in (0, 1, 3):
+        assert torch.equal(run_abi(Ai, layouts(Bi, b_layout), dev, b_layout, c_layout, v, group_m=gm), want)
+    ones = torch.ones(40, 1024, dtype=torch.bfloat16)
+    assert torch.all(run_abi(ones, layouts(torch.ones(1024, 264, dtype=torch.bfloat16), b_layout), dev, b_layout, c_layout, v) == 1024)
+
+
+@pytest.mark.parametrize("b_layout,c_layout", CHAIN_CELLS)
+def test_chain_kernel_k_loop_and_edges(dev, b_layout, c_layout):
+    """Period counts 1..9 and 16 (the loop body holds two periods; the prologue holds two tiles), ragged M and N (row
+    and column masks, two tile rows and columns), against the oracle and against the slab kernel bit for bit."""
+    for M, N in ((264, 392), (8, 16), (520, 528)):
+        for K in (128, 256, 384, 512, 640, 768, 896, 1024, 1152, 2048):
+            A, Bkn = o.make_inputs(M, N, K, seed=M + K)
+            B = layouts(Bkn, b_layout)
+            got = run_abi(A, B, dev, b_layout, c_layout, g.VARIANT_C256x256_W4)
+            o.assert_parity(got, A, Bkn, what=f"chain {M}x{N}x{K} b{b_layout} c{c_layout}")
+            assert torch.equal(got, run_abi(A, B, dev, b_layout, c_layout, g.VARIANT_T256x256_W4)), (M, N, K)
+
+
+def test_chain_kernel_refuses_what_it_cannot_run(dev):
+    A = torch.zeros(256, 512, dtype=torch.bfloat16, device=dev)
+    v = g.VARIANT_C256x256_W4
+    ws = torch.empty(4 * 256 * 256 * 4, dtype=torch.uint8, device=dev)
+    call = lambda K, b, c, split: _abi.gemm_raw(A.data_ptr(), A.data_ptr(), A.data_ptr(), 256, 256, K, 512, 512, 256, b, c,
+                                                ws.data_ptr(), ws.numel(), 0, v, split, 0)
+    assert call(256, g.B_NK, g.C_ROW, 1) == _abi.OK
+    assert call(192, g.B_NK, g.C_ROW, 1) == _abi.ERR_UNSUPPORTED     # K not in whole periods of 128
+    assert call(256, g.B_NK, g.C_ROW, 2) == _abi.ERR_UNSUPPORTED     # no split-K
+    assert call(256, g.B_KN, g.C_COL, 1) == _abi.ERR_UNSUPPORTED     # rows from an MN-major operand
+    torch.cuda.synchronize()
+    # the plan never sends such a problem there
+    assert g.plan(4096, 4096, 4096 + 64)[0] != v and g.plan(4096, 4096, 4096, g.B_KN, g.C_COL)[0] != v
+    assert g.plan(4096, 4096, 4096) == (v, 1) and g.plan(8192, 8192, 8192, g.B_NK, g.C_COL) == (v, 1)
+
+
 def test_variants_agree_bitwise_on_exact_data(dev):
     rng = np.random.default_rng(5)
     M, N, K = 512, 768, 384
