@@ -30,7 +30,7 @@ sys.path.insert(0, ROOT)
 PEAK_TFLOPS = 2500.0   # MI355X dense BF16
 PEAK_HBM_GBS = 8000.0  # MI355X HBM3E
 MATMUL_BENCH = os.path.join(ROOT, "gemm_amd", "vendor_bench", "matmul_bench")
-TRAFFIC_FILE = os.path.join(ROOT, "profiles", "gemm_tile_256x256_w4_8192cubed_traffic.json")
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "gemm_chain_256x256_8192cubed_traffic.json")
 
 
 def run_harness(args, env_extra=None, timeout=300):
