@@ -12,6 +12,7 @@
 #include <stdio.h>
 #include <stdlib.h>
 
+#include <atomic>
 #include <map>
 #include <mutex>
 #include <type_traits>
@@ -138,6 +139,7 @@ struct TileArgs {
   unsigned long long* prof;      // phase timers, 4 per wave (profiling instantiation only)
   float alpha, beta;             // C = alpha * A*B + beta * C (beta == 0: C is not read)
   long bsa, bsb, bsc;            // batch strides in elements; blockIdx.z is the batch index
+  int early_stores;              // gemm_chain_kernel: stage the epilogue a quarter wave tile at a time (see launch_chain)
   int batch;
 };
 
@@ -340,10 +342,12 @@ struct QuadMap {  // local 64-row / 64-column halves lie 128 apart (gemm_chain_k
 
 // Epilogue of the tile kernels: the TM x TN accumulator tiles of a wave (NW waves per workgroup, LDS_BYTES of LDS
 // that the main loop is done with) go to C as bf16, or to the split-K partials as fp32.
-template <int TM, int TN, int NW, uint32_t LDS_BYTES, class Map>
+// STAGE_TM: row tiles of the wave tile that go through LDS at a time (TM: all of it at once).
+template <int TM, int TN, int NW, uint32_t LDS_BYTES, int STAGE_TM = TM, class Map>
 __device__ __forceinline__ void store_wave_tile(f32x4 (&acc)[TM][TN], const TileArgs& p, char* gC, int kz, int lane,
                                                 int wave, uint32_t lds0, const Map map) {
   constexpr int WTM = TM * 16, WTN = TN * 16;
+  static_assert(TM % STAGE_TM == 0, "staging chunks are whole row tiles");
   // Epilogue: lane holds, per 16x16 tile, output row (lane & 15) and 4 consecutive columns 4*(lane >> 4)..+3.
   const int row_l = lane & 15, colq = (lane >> 4) * 4;
   // An accumulator element is read out of its AGPR where it is used: left to itself the compiler copies
@@ -370,45 +374,49 @@ __device__ __forceinline__ void store_wave_tile(f32x4 (&acc)[TM][TN], const Tile
       __builtin_amdgcn_s_barrier();
       asm volatile("" ::: "memory");
       const uint32_t region = lds0 + (uint32_t)wave * (WTM * WTN * 2);
-      auto park = [&](auto scaled) {
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-          const uint32_t row = i * 16 + row_l;
-#pragma unroll
-          for (int j = 0; j < TN; ++j) {
-            bf16x4 o;
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-              float v = acc_get(acc[i][j][r]);
-              if constexpr (decltype(scaled)::value) v *= p.alpha;
-              o[r] = (__bf16)v;
-            }
-            const uint32_t c = 2 * j + (lane >> 5);
-            const uint32_t addr = region + row * (WTN * 2) + ((c ^ (row & (CH - 1))) << 4) + (((lane >> 4) & 1) << 3);
-            *((NEOGEMM_AS3 bf16x4*)(uintptr_t)addr) = o;
-          }
-        }
-      };
-      if (p.alpha == 1.f) park(std::false_type{});
-      else park(std::true_type{});
-      // same wave wrote and reads: LDS operations of a wave complete in order; the compiler orders them
       const int colc = lane % CH;
       const int col = map.col(colc * 8);
 #pragma unroll
-      for (int st = 0; st < WTM / RPI; ++st) {
-        const uint32_t row = st * RPI + lane / CH;
-        const uint32_t addr = region + row * (WTN * 2) + (((uint32_t)colc ^ (row & (CH - 1))) << 4);
-        const bf16x8 v = *((NEOGEMM_AS3 bf16x8*)(uintptr_t)addr);
-        const int grow = map.row((int)row);
-        if (grow < p.M) {
-          char* dst = gC + ((size_t)grow * p.ldc + col) * 2;
-          if (col + 7 < p.N) {
-            // C is written once and not read again here: streaming stores leave the L2 to A and B
-            __builtin_nontemporal_store(v, (bf16x8*)dst);
-          } else {
+      for (int i0 = 0; i0 < TM; i0 += STAGE_TM) {
+        // rows i0*16 .. of the wave tile are rows 0 .. of the staging region
+        auto park = [&](auto scaled) {
 #pragma unroll
-            for (int e = 0; e < 8; ++e)
-              if (col + e < p.N) ((__bf16*)dst)[e] = v[e];
+          for (int i = i0; i < i0 + STAGE_TM; ++i) {
+            const uint32_t row = (i - i0) * 16 + row_l;
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+              bf16x4 o;
+#pragma unroll
+              for (int r = 0; r < 4; ++r) {
+                float v = acc_get(acc[i][j][r]);
+                if constexpr (decltype(scaled)::value) v *= p.alpha;
+                o[r] = (__bf16)v;
+              }
+              const uint32_t c = 2 * j + (lane >> 5);
+              const uint32_t addr = region + row * (WTN * 2) + ((c ^ (row & (CH - 1))) << 4) + (((lane >> 4) & 1) << 3);
+              *((NEOGEMM_AS3 bf16x4*)(uintptr_t)addr) = o;
+            }
+          }
+        };
+        if (p.alpha == 1.f) park(std::false_type{});
+        else park(std::true_type{});
+        // same wave wrote and reads: LDS operations of a wave complete in order; the compiler orders them
+#pragma unroll
+        for (int st = 0; st < STAGE_TM * 16 / RPI; ++st) {
+          const uint32_t row = st * RPI + lane / CH;
+          const uint32_t addr = region + row * (WTN * 2) + (((uint32_t)colc ^ (row & (CH - 1))) << 4);
+          const bf16x8 v = *((NEOGEMM_AS3 bf16x8*)(uintptr_t)addr);
+          const int grow = map.row(i0 * 16 + (int)row);
+          if (grow < p.M) {
+            char* dst = gC + ((size_t)grow * p.ldc + col) * 2;
+            if (col + 7 < p.N) {
+              // C is written once and not read again here: streaming stores leave the L2 to A and B
+              __builtin_nontemporal_store(v, (bf16x8*)dst);
+            } else {
+#pragma unroll
+              for (int e = 0; e < 8; ++e)
+                if (col + e < p.N) ((__bf16*)dst)[e] = v[e];
+            }
           }
         }
       }
@@ -1064,17 +1072,32 @@ __global__ __launch_bounds__(256) void gemm_chain_kernel(TileArgs p) {
   for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int jn = 0; jn < TN; ++jn) asm volatile("" : "+a"(acc[i][jn]));
-  store_wave_tile<TM, TN, NW, LDS_BYTES>(acc, p, gC, kz, lane, wave, lds0, BlockMap{m0 + wm * 128, n0 + wn * 128});
+  // With one round of workgroups the whole chip reaches its epilogue at once and nothing overlaps it: staging a quarter
+  // of the wave tile at a time gets the first stores on their way after a quarter of the conversions (4096^3 and
+  // 3000x5120x3584: -0.5 %); with several rounds the plain staging is 0.5 % ahead (8192^3).
+  if (p.early_stores) store_wave_tile<TM, TN, NW, LDS_BYTES, TM / 4>(acc, p, gC, kz, lane, wave, lds0, BlockMap{m0 + wm * 128, n0 + wn * 128});
+  else store_wave_tile<TM, TN, NW, LDS_BYTES>(acc, p, gC, kz, lane, wave, lds0, BlockMap{m0 + wm * 128, n0 + wn * 128});
 }
 
 hipError_t launch_chain(const TileArgs& a, bool bk, hipStream_t st);
 #if NEOGEMM_HAS_PART(8)
 hipError_t launch_chain(const TileArgs& a, bool bk, hipStream_t st) {
   const size_t lds = 5 * 32768;
+  // one round of workgroups or several (one workgroup per CU)
+  static std::atomic<int> cus_of[64];
+  int dev = 0;
+  if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
+  int cus = dev >= 0 && dev < 64 ? cus_of[dev].load(std::memory_order_relaxed) : 0;
+  if (cus == 0) {
+    if (hipError_t e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev); e != hipSuccess) return e;
+    if (dev >= 0 && dev < 64) cus_of[dev].store(cus, std::memory_order_relaxed);
+  }
+  TileArgs b = a;
+  b.early_stores = (int64_t)a.ntm * a.ntn * a.batch <= cus;
   dim3 grid(a.ntm * a.ntn, 1, a.batch), block(256);
   auto go = [&](auto kern) -> hipError_t {
     if (hipError_t e = allow_lds(kern, lds); e != hipSuccess) return e;
-    kern<<<grid, block, lds, st>>>(a);
+    kern<<<grid, block, lds, st>>>(b);
     return hipGetLastError();
   };
   return bk ? go(gemm_chain_kernel<true>) : go(gemm_chain_kernel<false>);
@@ -1792,6 +1815,7 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
   a.ws = nullptr;
   a.prof = prof;
   a.alpha = alpha;
+  a.early_stores = 0;
   a.beta = beta;
   if (prof && (bt.count > 1 || a.ksplit > 1 || vi.bm != 256 || vi.bn != 256 || !ak || v == NEOGEMM_VARIANT_C256x256_W4))
     return NEOGEMM_ERR_UNSUPPORTED;
