@@ -26,17 +26,28 @@ CANDIDATE_VARIANTS = (_abi.VARIANT_T256x256_W4, _abi.VARIANT_C256x256_W4, _abi.V
 CANDIDATE_SPLITS = (1, 2, 3, 4, 6, 8, 12, 16, 24, 32)
 
 
-def time_us(fn, warmup=5, iters=30):
+def time_us(fn, warmup=5, iters=30, preheat_ms=0.0):
+    """Microseconds per call: median of three event-bracketed batches, after `warmup` calls and, for launches long
+    enough to be power-limited, `preheat_ms` of the same call (the first launches after an idle stretch run on clocks
+    that have not settled: an 8192^3 GEMM takes 15 % longer there)."""
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    start.record()
-    for _ in range(iters):
-        fn()
-    stop.record()
-    stop.synchronize()
-    return start.elapsed_time(stop) * 1000.0 / iters
+
+    def batch(n):
+        start.record()
+        for _ in range(n):
+            fn()
+        stop.record()
+        stop.synchronize()
+        return start.elapsed_time(stop) * 1000.0 / n
+
+    heated = 0.0
+    while heated < preheat_ms * 1000.0:
+        heated += batch(10) * 10
+    per = max(1, iters // 3)
+    return sorted(batch(per) for _ in range(3))[1]
 
 
 def tune_shape(M, N, K, nbuf=1, log=sys.stderr, b_layout=B_KN, c_layout=C_ROW):
@@ -53,21 +64,22 @@ def tune_shape(M, N, K, nbuf=1, log=sys.stderr, b_layout=B_KN, c_layout=C_ROW):
         gemm_into(A, Bs[turn[0] % nbuf], C, M, N, K, K, b_shape[1], C.shape[1], b_layout, c_layout, variant, split, 0)
 
     model = plan(M, N, K, b_layout, c_layout)
-    t_model = time_us(lambda: call(None, 0))
+    heat = 150.0 if 2.0 * M * N * K > 5e10 else 0.0   # GEMMs of tens of microseconds and more run into the power limit
+    t_model = time_us(lambda: call(None, 0), preheat_ms=heat)
     best, t_best = model, t_model
     for v in CANDIDATE_VARIANTS:
         for s in CANDIDATE_SPLITS:
             if s > 1 and K // (64 * s) < 2:
                 break
             try:
-                t = time_us(lambda: call(v, s))
+                t = time_us(lambda: call(v, s), preheat_ms=heat)
             except NeoGemmError as e:
                 if e.status != ERR_UNSUPPORTED:
                     raise
                 break
             if t < t_best:
                 best, t_best = (v, s), t
-    t_model = min(t_model, time_us(lambda: call(None, 0)))   # the first measurement ran on a cold clock
+    t_model = min(t_model, time_us(lambda: call(None, 0), preheat_ms=heat))   # the first measurement ran on a cold clock
     if best == model or t_model <= t_best:
         best, t_best = model, t_model
     print(f"{M}x{N}x{K} b{b_layout} c{c_layout}: model {model} {t_model:.2f} us, best {best} {t_best:.2f} us", file=log)
