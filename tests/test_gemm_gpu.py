@@ -329,12 +329,15 @@ def test_reference_call_contract(dev, modname):
     o.assert_parity(C3.view(N2, M2).t(), A2, B2, b_layout="nk", what=f"{modname}.neoGemmV1 non-square")
 
 
-@pytest.mark.parametrize("M,N,K", [(1024, 6144, 8192), (4096, 1536, 8192), (1024, 1024, 32768)])
+@pytest.mark.parametrize("M,N,K", [(1024, 6144, 8192), (4096, 1536, 8192), (1024, 1024, 32768), (3072, 1024, 16384)])
 def test_reference_call_on_split_k_shapes(dev, M, N, K):
     """neoGemmV1's layout (B [N,K], column-major C: nemgemmV03.cu:343-391) on shapes whose plan for that layout
-    splits K: both wrappers size the workspace with neogemm_bf16_workspace_bytes and the call must go through;
-    the raw C-ABI call with a workspace of exactly the queried size likewise."""
+    splits K, or did at some stage of the cost model (the first two: the cells where the workspace query once fell
+    short): both wrappers size the workspace with neogemm_bf16_workspace_bytes and the call must go through; the raw
+    C-ABI call with a workspace of exactly the queried size likewise."""
     import neoGEMM
+    if (M, N, K) in ((1024, 1024, 32768), (3072, 1024, 16384)):
+        assert g.plan(M, N, K, g.B_NK, g.C_COL)[1] > 1
     A, Bnk = o.make_inputs(M, N, K, seed=M + N, b_layout="nk")
     Ad, Bd = A.to(dev), Bnk.to(dev)
     ref = o.ref_gemm(A, Bnk, b_layout="nk")
