@@ -6,7 +6,9 @@
 // with TMA and issues WGMMA from one warpgroup (v01.cu:215-237); here a workgroup of wave64s owns a
 // 256x256 (or smaller) macro-tile, stages K with direct-to-LDS buffer loads into a ring of three or four
 // XOR-swizzled LDS images per operand (64-deep tiles of a K-major operand, 32-deep slabs of an MN-major
-// one), and feeds v_mfma_f32_16x16x32_bf16 from ds_read_b128 / ds_read_b64_tr_b16.
+// one), and feeds v_mfma_f32_16x16x32_bf16 from ds_read_b128 / ds_read_b64_tr_b16.  The large unsplit shapes run a
+// second 256x256 kernel (gemm_chain_kernel) that issues both K steps of an accumulator tile back to back: same sums in
+// the same order, less power per MFMA on a chip whose clock is set by its power limit.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stdio.h>
@@ -25,7 +27,7 @@
 // Split build: compiling this one file takes minutes because of the many instances of the tile kernel, so setup.py
 // compiles it NEOGEMM_PARTS times in parallel with -DNEOGEMM_PART=0..NEOGEMM_PARTS-1 and links the objects.  Part 0
 // holds everything but the tile kernels; part k > 0 instantiates its share of launch_tile<> (listed behind
-// launch_tile) and nothing else.  Without NEOGEMM_PART the file is one self-contained translation unit.
+// launch_tile) or, the last one, launch_chain, and nothing else.  Without NEOGEMM_PART the file is one self-contained translation unit.
 #ifdef NEOGEMM_PART
 #define NEOGEMM_HAS_PART(p) (NEOGEMM_PART == (p))
 #else
