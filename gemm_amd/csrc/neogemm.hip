@@ -1170,8 +1170,13 @@ namespace neogemm {
 // no barrier until the end, when the four partial sums meet in LDS and are added in wave order.
 // One step of one wave: A 16*TMF rows x 128 B (K-major image, swz_k), B 64 k-rows x 128 B if B is [K,N]
 // (64 columns are one cache line per k-row; swizzle swz_mn64) or 64 rows x 128 B if B is [N,K].
-// 4 waves x RS steps x (2 KiB * TMF + 8 KiB) of LDS: TMF = 1, RS = 4 fills the 160 KiB; TMF = 2, RS = 3 and
-// TMF = 4, RS = 2 (M <= 64: 30.5 us at 64x14336x4096, the split-K tile path 32.9) are the other instances.
+// 4 waves x (RA steps of A at 2 KiB * TMF + RS steps of B at 8 KiB) of LDS: TMF = 1 with rings of 4 fills the 160 KiB;
+// TMF = 2 with 3 and TMF = 4 with 2 (M <= 64: 30.5 us at 64x14336x4096, the split-K tile path 32.9) are the other
+// instances for up to 64 rows.  TMF = 5 .. 8 (up to 128 rows) fit two steps of each at most, or one of A and three of B.
+// A wave's loads complete in the order it issued them, so a ring deeper than the other operand's buys little: with one
+// step of A, B's third step shortens 96 x 14336 x 4096 by 3 % where a second step of A shortens it by 6 %.
+// (Fetching the fragments straight into registers instead, which would hold three steps of both, was slower by 40 %:
+// a fragment load touches 16 rows x 64 bytes, half a line each, and the vector L1 charges by the line.)
 // ---------------------------------------------------------------------------------------------
 __device__ __forceinline__ uint32_t swz_mn64(uint32_t kk) {
   // k-row kk (0..31 within a slab) of a 64-column MN-major image: even values 0..6 XOR-ed into the 16-byte chunk
@@ -1186,19 +1191,66 @@ struct SkinnyArgs {
   long lda, ldb, ldc;
   float alpha, beta;
 };
-template <int TMF, int RS, bool BKM, bool CCOL = false>
+// The end of the skinny kernels: the partial sums of the four waves (each over its share of K) meet in LDS (16 KiB * TMF
+// from `smem` on, which no wave may still be using) and wave w adds up fragment column w in wave order, scales and stores.
+template <int TMF, bool CCOL>
+__device__ __forceinline__ void skinny_reduce_store(f32x4 (&acc)[TMF][4], const SkinnyArgs& p, int n0, int wave, int lane,
+                                                    char* smem) {
+  const uint32_t frow = lane & 15, fq = (uint32_t)lane >> 4;
+  NEOGEMM_AS3 f32x4* red = (NEOGEMM_AS3 f32x4*)smem;
+#pragma unroll
+  for (int t = 0; t < TMF; ++t)
+#pragma unroll
+    for (int f = 0; f < 4; ++f) red[((wave * TMF + t) * 4 + f) * 64 + lane] = acc[t][f];
+  __syncthreads();
+#pragma unroll
+  for (int t = 0; t < TMF; ++t) {
+    f32x4 sum = red[((0 * TMF + t) * 4 + wave) * 64 + lane];
+#pragma unroll
+    for (int w = 1; w < 4; ++w) {
+      const f32x4 v = red[((w * TMF + t) * 4 + wave) * 64 + lane];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) sum[r] += v[r];
+    }
+    // the lane's four elements are consecutive along `fast` (n for a row-major C, m for a column-major one)
+    const int row = CCOL ? 16 * t + 4 * (int)fq : 16 * t + (int)frow;
+    const int col = CCOL ? n0 + 16 * wave + (int)frow : n0 + 16 * wave + 4 * (int)fq;
+    if (row >= p.M || col >= p.N) continue;
+    const int fast = CCOL ? row : col, fast_end = CCOL ? p.M : p.N;
+    char* cp = p.C + (CCOL ? (size_t)col * p.ldc + row : (size_t)row * p.ldc + col) * 2;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) sum[r] *= p.alpha;
+    if (p.beta != 0.f) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (fast + r < fast_end) sum[r] = __builtin_fmaf(p.beta, (float)((const __bf16*)cp)[r], sum[r]);
+    }
+    const bf16x4 o = {(__bf16)sum[0], (__bf16)sum[1], (__bf16)sum[2], (__bf16)sum[3]};
+    if (fast + 3 < fast_end) {
+      *(bf16x4*)cp = o;
+    } else {
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (fast + r < fast_end) ((__bf16*)cp)[r] = o[r];
+    }
+  }
+}
+
+template <int TMF, int RS, bool BKM, bool CCOL = false, int RA = RS>
 __global__ __launch_bounds__(256) void gemm_skinny_kernel(SkinnyArgs p) {
   constexpr int BM = 16 * TMF;
-  constexpr uint32_t A_STEP = BM * 128, B_STEP = 64 * 128, STEP = A_STEP + B_STEP;
+  constexpr uint32_t A_STEP = BM * 128, B_STEP = 64 * 128, WAVE_LDS = RA * A_STEP + RS * B_STEP;
   constexpr int NA = A_STEP / 1024, NB = B_STEP / 1024, LP = NA + NB;  // 1 KiB loads per step
-  static_assert(4u * RS * STEP <= 160u * 1024u, "the four rings must fit the LDS");
+  static_assert(RA >= 1 && RA <= RS, "A comes from L2 (every workgroup reads all of it): its ring may be the shorter one");
+  static_assert(4u * WAVE_LDS <= 160u * 1024u, "the four waves' rings must fit the LDS");
+  static_assert(4u * TMF * 4u * 64u * 16u <= 4u * WAVE_LDS, "the rings double as the reduction buffer");
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   const uint32_t lds0 = (uint32_t)(uintptr_t)(NEOGEMM_AS3 char*)smem;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n0 = blockIdx.x * 64;
   const int nsteps = (p.K + KTILE - 1) / KTILE;
-  const uint32_t ring = lds0 + (uint32_t)wave * RS * STEP;
+  const uint32_t ring_a = lds0 + (uint32_t)wave * WAVE_LDS, ring_b = ring_a + RA * A_STEP;
 
   // per-lane byte offsets of the loads of one step, relative to the step's first element of A / B; a load
   // carries the instruction offset (j & 3) * 1024 (see Operand::init), OOB_OFFSET where nothing is to be read
@@ -1237,14 +1289,12 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(SkinnyArgs p) {
     r[3] = 0x00020000;
     return r;
   };
-  // all loads of step s of this wave into ring slot `slot`; past K everything is masked (the loads are
-  // still issued, as zero fills, so that the count of loads in flight does not depend on K)
-  auto issue_step = [&](int s, int slot) {
+  // all loads of A / of B of step s of this wave into slot `slot` of that operand's ring; past K everything is
+  // masked (the loads are still issued, as zero fills, so that the count of loads in flight does not depend on K)
+  auto issue_a = [&](int s, int slot) {
     const int krem = s < s_end ? p.K - s * KTILE : 0;  // depth left from this step on (<= 0: nothing)
-    const uint32_t dst = ring + (uint32_t)slot * STEP;
+    const uint32_t dst = ring_a + (uint32_t)slot * A_STEP;
     const i32x4 ra = rsrc((uint64_t)p.A + (uint64_t)s * KTILE * 2);
-    const i32x4 rb = rsrc((uint64_t)p.B + (BKM ? ((uint64_t)n0 * p.ldb + (uint64_t)s * KTILE) * 2
-                                                : ((uint64_t)s * KTILE * p.ldb + n0) * 2));
     static_for<NA>([&](auto jc) {
       constexpr int j = decltype(jc)::value;
       uint32_t v = voa[j];
@@ -1253,6 +1303,12 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(SkinnyArgs p) {
       if constexpr (j % 4 == 0) dma_set_m0(dst + (j / 4) * 4096);
       dma16<(j & 3) * 1024>(ra, v);
     });
+  };
+  auto issue_b = [&](int s, int slot) {
+    const int krem = s < s_end ? p.K - s * KTILE : 0;
+    const uint32_t dst = ring_b + (uint32_t)slot * B_STEP;
+    const i32x4 rb = rsrc((uint64_t)p.B + (BKM ? ((uint64_t)n0 * p.ldb + (uint64_t)s * KTILE) * 2
+                                                : ((uint64_t)s * KTILE * p.ldb + n0) * 2));
     static_for<NB>([&](auto jc) {
       constexpr int j = decltype(jc)::value;
       uint32_t v = vob[j];
@@ -1263,7 +1319,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(SkinnyArgs p) {
       } else {
         if ((int)r >= krem) v = OOB_OFFSET;
       }
-      if constexpr (j % 4 == 0) dma_set_m0(dst + A_STEP + (j / 4) * 4096);
+      if constexpr (j % 4 == 0) dma_set_m0(dst + (j / 4) * 4096);
       dma16<(j & 3) * 1024>(rb, v);
     });
   };
@@ -1278,41 +1334,46 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(SkinnyArgs p) {
 
   // fragment addresses within a step image (see FragReader)
   const uint32_t frow = lane & 15, fq = (uint32_t)lane >> 4;
-  uint32_t a_off[2], b_off[2];
+  uint32_t a_off[2];  // B [N,K]: the same image shape, 64 rows
 #pragma unroll
-  for (int sl = 0; sl < 2; ++sl) {
-    a_off[sl] = frow * 128 + (((4 * sl + fq) ^ swz_k(frow)) << 4);
-    b_off[sl] = A_STEP + a_off[sl];  // B [N,K]: the same image shape, 64 rows
-  }
+  for (int sl = 0; sl < 2; ++sl) a_off[sl] = frow * 128 + (((4 * sl + fq) ^ swz_k(frow)) << 4);
   const uint32_t tr_r = frow >> 2, tr_c = frow & 3, kk = 8 * fq + tr_r;  // B [K,N]: k-row within a slab, the second read adds 4
 
-#pragma unroll
-  for (int r = 0; r < RS; ++r) issue_step(s_begin + s_stride * r, r);
-  int slot = 0;
+  // Trip t of the loop asks for A of step t + RA, then for B of step t + RS; the prologue is trips -RS .. -1 of that
+  // order.  At the top of trip t everything up to A of step t must have landed: behind it in the queue are the B loads
+  // issued in the same trip as that A (none if RA == RS: that B is step t's own) and RA - 1 whole trips.
+  static_for<RS>([&](auto rc) {
+    constexpr int r = decltype(rc)::value;
+    if constexpr (r + RA >= RS) issue_a(s_begin + s_stride * (r + RA - RS), r + RA - RS);
+    issue_b(s_begin + s_stride * r, r);
+  });
+  int slot_a = 0, slot_b = 0;
   for (int s = s_begin; s < s_end; s += s_stride) {
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((RS - 1) * LP) : "memory");
-    const uint32_t img = ring + (uint32_t)slot * STEP;
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((RA - 1) * LP + (RA < RS ? NB : 0)) : "memory");
+    const uint32_t img_a = ring_a + (uint32_t)slot_a * A_STEP, img_b = ring_b + (uint32_t)slot_b * B_STEP;
     bf16x8 af[2][TMF], bf[2][4];
 #pragma unroll
     for (int sl = 0; sl < 2; ++sl) {
 #pragma unroll
-      for (int t = 0; t < TMF; ++t) af[sl][t] = lds_read_b128(img + a_off[sl] + t * 2048);
+      for (int t = 0; t < TMF; ++t) af[sl][t] = lds_read_b128(img_a + a_off[sl] + t * 2048);
 #pragma unroll
       for (int f = 0; f < 4; ++f) {
         if constexpr (BKM) {
-          bf[sl][f] = lds_read_b128(img + b_off[sl] + f * 2048);
+          bf[sl][f] = lds_read_b128(img_b + a_off[sl] + f * 2048);
         } else {
           const uint32_t chunk = (2 * f + (tr_c >> 1)) ^ swz_mn64(kk);
-          const uint32_t ad = img + A_STEP + (32 * sl + kk) * 128 + (chunk << 4) + ((tr_c & 1) << 3);
+          const uint32_t ad = img_b + (32 * sl + kk) * 128 + (chunk << 4) + ((tr_c & 1) << 3);
           const i16x4 lo = lds_read_tr16(ad), hi = lds_read_tr16(ad + 4 * 128);
           bf[sl][f] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
         }
       }
     }
-    // the fragments must be in registers before the next loads overwrite this slot
+    // the fragments must be in registers before the next loads overwrite these slots
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    issue_step(s + s_stride * RS, slot);
-    slot = slot + 1 == RS ? 0 : slot + 1;
+    issue_a(s + s_stride * RA, slot_a);
+    issue_b(s + s_stride * RS, slot_b);
+    slot_a = slot_a + 1 == RA ? 0 : slot_a + 1;
+    slot_b = slot_b + 1 == RS ? 0 : slot_b + 1;
 #pragma unroll
     for (int sl = 0; sl < 2; ++sl)
 #pragma unroll
@@ -1327,44 +1388,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(SkinnyArgs p) {
   // drain the loads still in flight (zero fills past K included) before the rings become the reduction buffer
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
-  // partial sums of the four waves -> LDS; wave w then sums and writes fragment column w, in wave order
-  NEOGEMM_AS3 f32x4* red = (NEOGEMM_AS3 f32x4*)smem;
-#pragma unroll
-  for (int t = 0; t < TMF; ++t)
-#pragma unroll
-    for (int f = 0; f < 4; ++f) red[((wave * TMF + t) * 4 + f) * 64 + lane] = acc[t][f];
-  __syncthreads();
-#pragma unroll
-  for (int t = 0; t < TMF; ++t) {
-    f32x4 sum = red[((0 * TMF + t) * 4 + wave) * 64 + lane];
-#pragma unroll
-    for (int w = 1; w < 4; ++w) {
-      const f32x4 v = red[((w * TMF + t) * 4 + wave) * 64 + lane];
-#pragma unroll
-      for (int r = 0; r < 4; ++r) sum[r] += v[r];
-    }
-    // the lane's four elements are consecutive along `fast` (n for a row-major C, m for a column-major one)
-    const int row = CCOL ? 16 * t + 4 * (int)fq : 16 * t + (int)frow;
-    const int col = CCOL ? n0 + 16 * wave + (int)frow : n0 + 16 * wave + 4 * (int)fq;
-    if (row >= p.M || col >= p.N) continue;
-    const int fast = CCOL ? row : col, fast_end = CCOL ? p.M : p.N;
-    char* cp = p.C + (CCOL ? (size_t)col * p.ldc + row : (size_t)row * p.ldc + col) * 2;
-#pragma unroll
-    for (int r = 0; r < 4; ++r) sum[r] *= p.alpha;
-    if (p.beta != 0.f) {
-#pragma unroll
-      for (int r = 0; r < 4; ++r)
-        if (fast + r < fast_end) sum[r] = __builtin_fmaf(p.beta, (float)((const __bf16*)cp)[r], sum[r]);
-    }
-    const bf16x4 o = {(__bf16)sum[0], (__bf16)sum[1], (__bf16)sum[2], (__bf16)sum[3]};
-    if (fast + 3 < fast_end) {
-      *(bf16x4*)cp = o;
-    } else {
-#pragma unroll
-      for (int r = 0; r < 4; ++r)
-        if (fast + r < fast_end) ((__bf16*)cp)[r] = o[r];
-    }
-  }
+  skinny_reduce_store<TMF, CCOL>(acc, p, n0, wave, lane, smem);
 }
 
 // Sum the split-K partials in split order (deterministic) and round once to bf16.
@@ -1458,7 +1482,7 @@ struct VariantInfo {
 };
 static const VariantInfo kVariants[NEOGEMM_VARIANT_COUNT] = {
     {0, 0, 0}, {16, 16, 4}, {256, 256, 8}, {256, 256, 4}, {128, 128, 4}, {256, 128, 4}, {128, 256, 4}, {64, 128, 4}, {128, 128, 4},
-    {16, 64, 4}, {32, 64, 4}, {64, 64, 4}, {192, 256, 4}, {96, 128, 4}, {64, 64, 4}, {256, 256, 4},
+    {16, 64, 4}, {32, 64, 4}, {64, 64, 4}, {192, 256, 4}, {96, 128, 4}, {64, 64, 4}, {256, 256, 4}, {128, 64, 4},
 };
 
 static bool is_aligned(const void* A, const void* B, const void* C, int64_t K, int64_t lda, int64_t ldb,
@@ -1559,6 +1583,26 @@ static void plan_model(int64_t M, int64_t N, int64_t K, bool aligned, int c_layo
     if (t < best) {
       best = t;
       bv = rows <= 16 ? NEOGEMM_VARIANT_SKINNY16 : rows <= 32 ? NEOGEMM_VARIANT_SKINNY32 : NEOGEMM_VARIANT_SKINNY64;
+      bs = 1;
+    }
+  }
+  // 65 to 128 rows (of M, or of N with B [N,K]): the same kernel with five to eight row fragments per wave.  Its rings
+  // hold two steps at most then, so it is only the better choice where one round of strips about fills the CUs and K
+  // is a few thousand deep (decode shapes like 128 x 14336 x 4096: 36.1 us against 39.5 for split-K tiles with B [N,K];
+  // with B [K,N] 39.4 against 36.9 at 128 rows, 37.5 against 41.2 at 112).  Fitted to such timings; the tile estimates
+  // above come out about an eighth below what those shapes measure, hence the factor.
+  const bool wide_m = !skinny_m && !skinny_n && M <= 128;
+  const bool wide_n = !skinny_m && !skinny_n && !wide_m && N <= 128 && b_layout == NEOGEMM_B_NK;
+  if ((wide_m || wide_n) && batch == 1 && K >= 2048) {
+    const int64_t rows = wide_m ? M : N, cols = wide_m ? N : M;
+    const double wgs = (double)ceil_div(cols, 64), full = __builtin_floor(wgs / cus), frac = wgs / cus - full;
+    const double rounds = full + (frac > 0.0 ? 0.7 + 0.3 * frac : 0.0);
+    const double wg_bytes = (double)K * 128.0 + (double)ceil_div(rows, 16) * 16.0 * K * 2.0;
+    double t = 7.0 + rounds * wg_bytes / (b_layout == NEOGEMM_B_NK ? 52.0e3 : 46.0e3);
+    if (t < stream_us) t = stream_us;
+    if (t < best * 1.12) {
+      best = t;
+      bv = NEOGEMM_VARIANT_SKINNY128;
       bs = 1;
     }
   }
@@ -1726,7 +1770,8 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
 
   if (!aligned) return NEOGEMM_ERR_UNSUPPORTED;
 
-  if (v == NEOGEMM_VARIANT_SKINNY16 || v == NEOGEMM_VARIANT_SKINNY32 || v == NEOGEMM_VARIANT_SKINNY64) {
+  if (v == NEOGEMM_VARIANT_SKINNY16 || v == NEOGEMM_VARIANT_SKINNY32 || v == NEOGEMM_VARIANT_SKINNY64 ||
+      v == NEOGEMM_VARIANT_SKINNY128) {
     // what the skinny kernel assumes: M within its rows, whole 16-byte chunks of B [K,N] inside the matrix,
     // one problem.  If M is too large but N fits and B is [N,K], it runs the transposed problem
     // C^T = B * A^T: its small operand is B then, its wide one A, and the layout of C flips.
@@ -1755,17 +1800,26 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
       kern<<<dim3(ceil_div(sa.N, 64)), 256, lds, st>>>(sa);
       return hipGetLastError();
     };
-    auto pick = [&](auto tmf, auto rs) -> hipError_t {
-      constexpr int TMF = decltype(tmf)::value, RS = decltype(rs)::value;
-      constexpr size_t lds = (size_t)4 * RS * (TMF * 2048 + 8192);
-      if (bkm) return ccol ? go(gemm_skinny_kernel<TMF, RS, true, true>, lds) : go(gemm_skinny_kernel<TMF, RS, true, false>, lds);
-      return ccol ? go(gemm_skinny_kernel<TMF, RS, false, true>, lds) : go(gemm_skinny_kernel<TMF, RS, false, false>, lds);
+    auto pick = [&](auto tmf, auto rs, auto ra) -> hipError_t {
+      constexpr int TMF = decltype(tmf)::value, RS = decltype(rs)::value, RA = decltype(ra)::value;
+      constexpr size_t lds = (size_t)4 * (RA * TMF * 2048 + RS * 8192);
+      if (bkm) return ccol ? go(gemm_skinny_kernel<TMF, RS, true, true, RA>, lds) : go(gemm_skinny_kernel<TMF, RS, true, false, RA>, lds);
+      return ccol ? go(gemm_skinny_kernel<TMF, RS, false, true, RA>, lds) : go(gemm_skinny_kernel<TMF, RS, false, false, RA>, lds);
     };
     using std::integral_constant;
     hipError_t e;
-    if (v == NEOGEMM_VARIANT_SKINNY16) e = pick(integral_constant<int, 1>{}, integral_constant<int, 4>{});
-    else if (v == NEOGEMM_VARIANT_SKINNY32) e = pick(integral_constant<int, 2>{}, integral_constant<int, 3>{});
-    else e = pick(integral_constant<int, 4>{}, integral_constant<int, 2>{});
+    using I1 = integral_constant<int, 1>;
+    using I2 = integral_constant<int, 2>;
+    using I3 = integral_constant<int, 3>;
+    using I4 = integral_constant<int, 4>;
+    if (v == NEOGEMM_VARIANT_SKINNY16) e = pick(I1{}, I4{}, I4{});
+    else if (v == NEOGEMM_VARIANT_SKINNY32) e = pick(I2{}, I3{}, I3{});
+    else if (v == NEOGEMM_VARIANT_SKINNY64) e = pick(I4{}, I2{}, I2{});
+    // 65 to 128 rows, in sixteens: two steps of A and of B in the rings while they fit, else one of A and three of B
+    else if (sa.M <= 80) e = pick(integral_constant<int, 5>{}, I2{}, I2{});
+    else if (sa.M <= 96) e = pick(integral_constant<int, 6>{}, I2{}, I2{});
+    else if (sa.M <= 112) e = pick(integral_constant<int, 7>{}, I3{}, I1{});
+    else e = pick(integral_constant<int, 8>{}, I3{}, I1{});
     if (e != hipSuccess) {
       fprintf(stderr, "neogemm: skinny kernel launch failed (variant %d): %s\n", v, hipGetErrorString(e));
       return NEOGEMM_ERR_LAUNCH;

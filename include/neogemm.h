@@ -67,7 +67,10 @@ extern "C" {
    register-file traffic per flop: what the chip's power limit rewards); the operand that supplies the rows must be
    K-major, K a multiple of 128, no split-K. */
 #define NEOGEMM_VARIANT_C256x256_W4 15
-#define NEOGEMM_VARIANT_COUNT 16
+/* M <= 128 by the same kernel (five to eight row fragments of 16 per wave, shorter rings): one launch, no workspace;
+   chosen where one round of strips about fills the CUs and K is a few thousand deep */
+#define NEOGEMM_VARIANT_SKINNY128 16
+#define NEOGEMM_VARIANT_COUNT 17
 
 /*
  * C = A * op(B), bf16 in, fp32 accumulate, bf16 out.

@@ -195,7 +195,7 @@ def test_parity_8192_headline(dev):
     check_big(dev, 8192, 8192, 8192, seed=2)
 
 
-@pytest.mark.parametrize("M", [16, 64, 128])
+@pytest.mark.parametrize("M", [16, 64, 72, 100, 128])
 @pytest.mark.parametrize("b_layout", [g.B_KN, g.B_NK])
 def test_parity_skinny(dev, M, b_layout):
     check_big(dev, M, 14336, 4096, seed=3 + M, b_layout=b_layout)
@@ -727,9 +727,9 @@ def test_batched_argument_checks(dev):
 
 
 # ------------------------------------------------------------------------------------------------
-# skinny-M streaming kernels (M <= 16 / 32 / 64, row-major C): forced and through the plan
+# skinny-M streaming kernels (M <= 16 / 32 / 64, and 128 as two row blocks): forced and through the plan
 # ------------------------------------------------------------------------------------------------
-SKINNY = [(g.VARIANT_SKINNY16, 16), (g.VARIANT_SKINNY32, 32), (g.VARIANT_SKINNY64, 64)]
+SKINNY = [(g.VARIANT_SKINNY16, 16), (g.VARIANT_SKINNY32, 32), (g.VARIANT_SKINNY64, 64), (g.VARIANT_SKINNY128, 128)]
 
 
 @pytest.mark.parametrize("variant,rows", SKINNY)
@@ -739,7 +739,8 @@ def test_skinny_kernels(dev, variant, rows, b_layout, c_layout):
     # K: one step, a partial step, fewer steps than the four waves, more than the ring, a K tail;
     # N: one strip, a ragged strip (N % 64, N % 8 == 0), many strips; M: 1, ragged, full
     for (M, N, K) in ((1, 64, 64), (rows, 200, 72), (rows - 3, 1000, 520), (rows - 4, 1000, 520), (rows, 4096, 1032),
-                      (5, 2048, 8200), (8, 2048, 8200), (rows, 64, 4096), (3, 72, 136), (rows, 14336, 512)):
+                      (5, 2048, 8200), (8, 2048, 8200), (rows, 64, 4096), (3, 72, 136), (rows, 14336, 512),
+                      (rows // 2 + 1, 520, 1032), (rows // 2 + 4, 1096, 264), (rows - 16, 8, 256)):
         A, Bkn = o.make_inputs(M, N, K, seed=M + N + K)
         try:
             got = run_abi(A, layouts(Bkn, b_layout), dev, b_layout, c_layout, variant, strict=True)
@@ -773,6 +774,7 @@ def test_skinny_known_answers_and_refusals(dev):
     # alpha/beta pass through
     assert g.plan(16, 14336, 4096)[0] == g.VARIANT_SKINNY16 and g.plan(64, 14336, 4096)[0] == g.VARIANT_SKINNY64
     assert g.plan(16, 14336, 4096, c_layout=g.C_COL)[0] == g.VARIANT_SKINNY16
+    assert g.plan(96, 14336, 4096)[0] == g.VARIANT_SKINNY128 and g.plan(128, 14336, 4096, b_layout=g.B_NK)[0] == g.VARIANT_SKINNY128
     M, N, K = 16, 4096, 2048
     A, Bkn = o.make_inputs(M, N, K, seed=2)
     C0 = torch.randn(M, N, generator=gen).to(torch.bfloat16)
