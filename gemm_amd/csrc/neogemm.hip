@@ -1081,11 +1081,8 @@ __global__ __launch_bounds__(256) void gemm_chain_kernel(TileArgs p) {
   else store_wave_tile<TM, TN, NW, LDS_BYTES>(acc, p, gC, kz, lane, wave, lds0, BlockMap{m0 + wm * 128, n0 + wn * 128});
 }
 
-hipError_t launch_chain(const TileArgs& a, bool bk, hipStream_t st);
-#if NEOGEMM_HAS_PART(8)
-hipError_t launch_chain(const TileArgs& a, bool bk, hipStream_t st) {
-  const size_t lds = 5 * 32768;
-  // one round of workgroups or several (one workgroup per CU)
+// CUs of the current device (the runtime is asked once per device)
+inline hipError_t current_device_cus(int* out) {
   static std::atomic<int> cus_of[64];
   int dev = 0;
   if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
@@ -1094,6 +1091,17 @@ hipError_t launch_chain(const TileArgs& a, bool bk, hipStream_t st) {
     if (hipError_t e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev); e != hipSuccess) return e;
     if (dev >= 0 && dev < 64) cus_of[dev].store(cus, std::memory_order_relaxed);
   }
+  *out = cus;
+  return hipSuccess;
+}
+
+hipError_t launch_chain(const TileArgs& a, bool bk, hipStream_t st);
+#if NEOGEMM_HAS_PART(8)
+hipError_t launch_chain(const TileArgs& a, bool bk, hipStream_t st) {
+  const size_t lds = 5 * 32768;
+  // one round of workgroups or several (one workgroup per CU)
+  int cus = 0;
+  if (hipError_t e = current_device_cus(&cus); e != hipSuccess) return e;
   TileArgs b = a;
   b.early_stores = (int64_t)a.ntm * a.ntn * a.batch <= cus;
   dim3 grid(a.ntm * a.ntn, 1, a.batch), block(256);
@@ -1190,33 +1198,36 @@ struct SkinnyArgs {
   int M, N, K;
   long lda, ldb, ldc;
   float alpha, beta;
+  int strip;  // columns of C per workgroup: 64, or with B [N,K] a smaller multiple of 8 that fills the CUs better
 };
 // The end of the skinny kernels: the partial sums of the four waves (each over its share of K) meet in LDS (16 KiB * TMF
 // from `smem` on, which no wave may still be using) and wave w adds up fragment column w in wave order, scales and stores.
-template <int TMF, bool CCOL>
-__device__ __forceinline__ void skinny_reduce_store(f32x4 (&acc)[TMF][4], const SkinnyArgs& p, int n0, int wave, int lane,
+template <int TMF, bool CCOL, int NF>
+__device__ __forceinline__ void skinny_reduce_store(f32x4 (&acc)[TMF][NF], const SkinnyArgs& p, int n0, int wave, int lane,
                                                     char* smem) {
   const uint32_t frow = lane & 15, fq = (uint32_t)lane >> 4;
   NEOGEMM_AS3 f32x4* red = (NEOGEMM_AS3 f32x4*)smem;
 #pragma unroll
   for (int t = 0; t < TMF; ++t)
 #pragma unroll
-    for (int f = 0; f < 4; ++f) red[((wave * TMF + t) * 4 + f) * 64 + lane] = acc[t][f];
+    for (int f = 0; f < NF; ++f) red[((wave * TMF + t) * NF + f) * 64 + lane] = acc[t][f];
   __syncthreads();
-#pragma unroll
-  for (int t = 0; t < TMF; ++t) {
-    f32x4 sum = red[((0 * TMF + t) * 4 + wave) * 64 + lane];
+  // fragment i = t * NF + f goes to wave i mod 4 (with four fragment columns: column w to wave w)
+  for (int i = wave; i < TMF * NF; i += 4) {
+    const int t = i / NF, f = i % NF;
+    f32x4 sum = red[i * 64 + lane];
 #pragma unroll
     for (int w = 1; w < 4; ++w) {
-      const f32x4 v = red[((w * TMF + t) * 4 + wave) * 64 + lane];
+      const f32x4 v = red[(w * TMF * NF + i) * 64 + lane];
 #pragma unroll
       for (int r = 0; r < 4; ++r) sum[r] += v[r];
     }
     // the lane's four elements are consecutive along `fast` (n for a row-major C, m for a column-major one)
     const int row = CCOL ? 16 * t + 4 * (int)fq : 16 * t + (int)frow;
-    const int col = CCOL ? n0 + 16 * wave + (int)frow : n0 + 16 * wave + 4 * (int)fq;
-    if (row >= p.M || col >= p.N) continue;
-    const int fast = CCOL ? row : col, fast_end = CCOL ? p.M : p.N;
+    const int col = CCOL ? n0 + 16 * f + (int)frow : n0 + 16 * f + 4 * (int)fq;
+    const int col_end = n0 + p.strip < p.N ? n0 + p.strip : p.N;  // a strip may be narrower than its fragments
+    if (row >= p.M || col >= col_end) continue;
+    const int fast = CCOL ? row : col, fast_end = CCOL ? p.M : col_end;
     char* cp = p.C + (CCOL ? (size_t)col * p.ldc + row : (size_t)row * p.ldc + col) * 2;
 #pragma unroll
     for (int r = 0; r < 4; ++r) sum[r] *= p.alpha;
@@ -1236,19 +1247,21 @@ __device__ __forceinline__ void skinny_reduce_store(f32x4 (&acc)[TMF][4], const 
   }
 }
 
-template <int TMF, int RS, bool BKM, bool CCOL = false, int RA = RS>
+template <int TMF, int RS, bool BKM, bool CCOL = false, int RA = RS, int SW = 64>
 __global__ __launch_bounds__(256) void gemm_skinny_kernel(SkinnyArgs p) {
-  constexpr int BM = 16 * TMF;
-  constexpr uint32_t A_STEP = BM * 128, B_STEP = 64 * 128, WAVE_LDS = RA * A_STEP + RS * B_STEP;
+  constexpr int BM = 16 * TMF, NF = SW / 16;  // rows of A, 16-column fragments of the strip
+  constexpr uint32_t A_STEP = BM * 128, B_STEP = SW * 128, WAVE_LDS = RA * A_STEP + RS * B_STEP;
   constexpr int NA = A_STEP / 1024, NB = B_STEP / 1024, LP = NA + NB;  // 1 KiB loads per step
+  static_assert(SW == 64 || (BKM && (SW == 32 || SW == 16)), "narrow strips only of a K-major B (whole lines per row)");
   static_assert(RA >= 1 && RA <= RS, "A comes from L2 (every workgroup reads all of it): its ring may be the shorter one");
   static_assert(4u * WAVE_LDS <= 160u * 1024u, "the four waves' rings must fit the LDS");
-  static_assert(4u * TMF * 4u * 64u * 16u <= 4u * WAVE_LDS, "the rings double as the reduction buffer");
+  static_assert(4u * TMF * NF * 64u * 16u <= 4u * WAVE_LDS, "the rings double as the reduction buffer");
+  static_assert((RA - 1) * LP + (RA < RS ? NB : 0) <= 63 && RA * NA + RS * NB <= 64, "the wait counts must fit the counter");
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   const uint32_t lds0 = (uint32_t)(uintptr_t)(NEOGEMM_AS3 char*)smem;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int n0 = blockIdx.x * 64;
+  const int n0 = blockIdx.x * p.strip;
   const int nsteps = (p.K + KTILE - 1) / KTILE;
   const uint32_t ring_a = lds0 + (uint32_t)wave * WAVE_LDS, ring_b = ring_a + RA * A_STEP;
 
@@ -1267,7 +1280,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(SkinnyArgs p) {
     if constexpr (BKM) {
       const uint32_t c = (lane & 7) ^ swz_k(r);
       vob[j] = r * (uint32_t)p.ldb * 2 + c * 16 + VOFF_BIAS - (j & 3) * 1024;
-      if (n0 + (int)r >= p.N) vob[j] = OOB_OFFSET;
+      if (n0 + (int)r >= p.N || (int)r >= p.strip) vob[j] = OOB_OFFSET;  // rows past the strip: still issued, as zero fills
     } else {
       const uint32_t c = (lane & 7) ^ swz_mn64(r & 31);
       vob[j] = r * (uint32_t)p.ldb * 2 + c * 16 + VOFF_BIAS - (j & 3) * 1024;
@@ -1324,11 +1337,11 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(SkinnyArgs p) {
     });
   };
 
-  f32x4 acc[TMF][4];
+  f32x4 acc[TMF][NF];
 #pragma unroll
   for (int t = 0; t < TMF; ++t)
 #pragma unroll
-    for (int f = 0; f < 4; ++f)
+    for (int f = 0; f < NF; ++f)
 #pragma unroll
       for (int v = 0; v < 4; ++v) acc[t][f][v] = 0.f;
 
@@ -1351,13 +1364,13 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(SkinnyArgs p) {
   for (int s = s_begin; s < s_end; s += s_stride) {
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"((RA - 1) * LP + (RA < RS ? NB : 0)) : "memory");
     const uint32_t img_a = ring_a + (uint32_t)slot_a * A_STEP, img_b = ring_b + (uint32_t)slot_b * B_STEP;
-    bf16x8 af[2][TMF], bf[2][4];
+    bf16x8 af[2][TMF], bf[2][NF];
 #pragma unroll
     for (int sl = 0; sl < 2; ++sl) {
 #pragma unroll
       for (int t = 0; t < TMF; ++t) af[sl][t] = lds_read_b128(img_a + a_off[sl] + t * 2048);
 #pragma unroll
-      for (int f = 0; f < 4; ++f) {
+      for (int f = 0; f < NF; ++f) {
         if constexpr (BKM) {
           bf[sl][f] = lds_read_b128(img_b + a_off[sl] + f * 2048);
         } else {
@@ -1379,7 +1392,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(SkinnyArgs p) {
 #pragma unroll
       for (int t = 0; t < TMF; ++t)
 #pragma unroll
-        for (int f = 0; f < 4; ++f)
+        for (int f = 0; f < NF; ++f)
           // B fragment first: a lane ends up with 4 consecutive n of one output row (see gemm_tile_kernel);
           // for a column-major C the other way round: 4 consecutive m of one output column
           if constexpr (CCOL) acc[t][f] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[sl][t], bf[sl][f], acc[t][f], 0, 0, 0);
@@ -1388,7 +1401,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(SkinnyArgs p) {
   // drain the loads still in flight (zero fills past K included) before the rings become the reduction buffer
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
-  skinny_reduce_store<TMF, CCOL>(acc, p, n0, wave, lane, smem);
+  skinny_reduce_store<TMF, CCOL, NF>(acc, p, n0, wave, lane, smem);
 }
 
 // Sum the split-K partials in split order (deterministic) and round once to bf16.
@@ -1567,20 +1580,33 @@ static void plan_model(int64_t M, int64_t N, int64_t K, bool aligned, int c_layo
       }
     }
   }
-  // the skinny-M streaming kernel: one strip of 64 columns and all of K per workgroup, 128 KiB
+  // the skinny-M streaming kernel: one strip of up to 64 columns and all of K per workgroup, 128 KiB
   // (M <= 16), 96 KiB (M <= 32) or 64 KiB (M <= 64) of B in flight each at ~2.5 us per round trip; no split-K,
   // one launch
   // With B [N,K] and N <= 64 < M the same kernel runs the transposed problem (the wide operand is A then).
   const bool skinny_m = M <= 64, skinny_n = !skinny_m && N <= 64 && b_layout == NEOGEMM_B_NK;
   if ((skinny_m || skinny_n) && batch == 1 && K >= 4 * KTILE) {
     const int64_t rows = skinny_m ? M : N, cols = skinny_m ? N : M;  // the kernel's own terms, whatever the layout of C
-    const double wgs = (double)ceil_div(cols, 64), full = __builtin_floor(wgs / cus), frac = wgs / cus - full;
-    const double rounds = full + (frac > 0.0 ? 0.7 + 0.3 * frac : 0.0);
-    const double wg_us = ((double)K * 128.0 + (double)rows * K * 2.0) / (rows <= 16 ? 51.0e3 : rows <= 32 ? 43.0e3 : 39.0e3);
-    double t = rounds * wg_us;
-    if (t < stream_us) t = stream_us;
+    double t;
+    if (b_layout == NEOGEMM_B_NK) {
+      // K-major wide operand: strips as wide as fills the CUs in whole rounds (see the launcher).  A workgroup pays
+      // for the bytes of its strip (from HBM) and, less, for those of the small operand (from L2); fitted to timings
+      // of 16 to 64 rows x 4096 .. 20480 columns x 4096 .. 14336 deep, all within 6 % but K = 8192 (-20 %).
+      const int rounds = ceil_div(ceil_div(cols, 64), (int64_t)cus);
+      int w = 8 * ceil_div(cols, 8 * (int64_t)rounds * (int64_t)cus);
+      w = w < 16 ? 16 : w > 64 ? 64 : w;
+      const double frags = (double)ceil_div(rows, 16) * 16.0;
+      t = (double)ceil_div(ceil_div(cols, w), (int64_t)cus) * ((double)w * K * 2.0 / 26.9e3 + frags * K * 2.0 / 90.0e3);
+      if (t < bytes / 5.9e6) t = bytes / 5.9e6;
+    } else {
+      const double wgs = (double)ceil_div(cols, 64), full = __builtin_floor(wgs / cus), frac = wgs / cus - full;
+      const double rounds = full + (frac > 0.0 ? 0.7 + 0.3 * frac : 0.0);
+      t = rounds * ((double)K * 128.0 + (double)rows * K * 2.0) / (rows <= 16 ? 51.0e3 : rows <= 32 ? 43.0e3 : 39.0e3);
+      if (t < stream_us) t = stream_us;
+    }
     t += 3.0;
-    if (t < best) {
+    // (the tile estimates come out a little low for shapes that stream from HBM with few rows, see below)
+    if (t < best * (b_layout == NEOGEMM_B_NK && bytes > 32e6 ? 1.04 : 1.0)) {
       best = t;
       bv = rows <= 16 ? NEOGEMM_VARIANT_SKINNY16 : rows <= 32 ? NEOGEMM_VARIANT_SKINNY32 : NEOGEMM_VARIANT_SKINNY64;
       bs = 1;
@@ -1788,16 +1814,30 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
                   NEOGEMM_VARIANT_GENERIC, 1, 0, nullptr, alpha, beta, bt);
       return st2;
     }
-    SkinnyArgs sa{(const char*)A, (const char*)B, (char*)C, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, alpha, beta};
+    SkinnyArgs sa{(const char*)A, (const char*)B, (char*)C, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, alpha, beta, 64};
     bool bkm = b_layout == NEOGEMM_B_NK, ccol = c_layout == NEOGEMM_C_COL;
     if (swap) {
-      sa = SkinnyArgs{(const char*)B, (const char*)A, (char*)C, (int)N, (int)M, (int)K, (long)ldb, (long)lda, (long)ldc, alpha, beta};
+      sa = SkinnyArgs{(const char*)B, (const char*)A, (char*)C, (int)N, (int)M, (int)K, (long)ldb, (long)lda, (long)ldc, alpha, beta, 64};
       bkm = true;    // A [M,K] takes the place of a B [N,K]
       ccol = !ccol;  // a row-major C[m][n] is the column-major C^T
     }
+    const bool wide = v == NEOGEMM_VARIANT_SKINNY128;
+    if (bkm) {
+      // A strip of a K-major B may start at any row of it and be of any width that is a multiple of 8: the width is
+      // chosen so that whole rounds of strips fill the CUs (N = 14336: 256 strips of 56 columns instead of 224 of 64,
+      // +1 to 3 %; N = 4096: 256 of 16 instead of 64 of 64, 50 -> 32 us at K = 14336 before the rings were deepened).
+      int cus = 0;
+      if (hipError_t e = current_device_cus(&cus); e != hipSuccess) {
+        fprintf(stderr, "neogemm: device query failed: %s\n", hipGetErrorString(e));
+        return NEOGEMM_ERR_LAUNCH;
+      }
+      const int rounds = ceil_div(ceil_div(sa.N, 64), cus), w = 8 * ceil_div(sa.N, 8 * (int64_t)rounds * cus);
+      if (w < 64 && w >= (wide ? 48 : 16)) sa.strip = w;
+      else if (w < 16 && !wide) sa.strip = 16;
+    }
     auto go = [&](auto kern, size_t lds) -> hipError_t {
       if (hipError_t e = allow_lds(kern, lds); e != hipSuccess) return e;
-      kern<<<dim3(ceil_div(sa.N, 64)), 256, lds, st>>>(sa);
+      kern<<<dim3(ceil_div(sa.N, sa.strip)), 256, lds, st>>>(sa);
       return hipGetLastError();
     };
     auto pick = [&](auto tmf, auto rs, auto ra) -> hipError_t {
@@ -1806,18 +1846,30 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
       if (bkm) return ccol ? go(gemm_skinny_kernel<TMF, RS, true, true, RA>, lds) : go(gemm_skinny_kernel<TMF, RS, true, false, RA>, lds);
       return ccol ? go(gemm_skinny_kernel<TMF, RS, false, true, RA>, lds) : go(gemm_skinny_kernel<TMF, RS, false, false, RA>, lds);
     };
+    // strips of at most 32 / 16 columns of a K-major B: smaller steps of B, deeper rings
+    auto pick_narrow = [&](auto tmf, auto rs, auto sw) -> hipError_t {
+      constexpr int TMF = decltype(tmf)::value, RS = decltype(rs)::value, SW = decltype(sw)::value;
+      constexpr size_t lds = (size_t)4 * RS * (TMF * 2048 + SW * 128);
+      return ccol ? go(gemm_skinny_kernel<TMF, RS, true, true, RS, SW>, lds) : go(gemm_skinny_kernel<TMF, RS, true, false, RS, SW>, lds);
+    };
     using std::integral_constant;
     hipError_t e;
     using I1 = integral_constant<int, 1>;
     using I2 = integral_constant<int, 2>;
     using I3 = integral_constant<int, 3>;
     using I4 = integral_constant<int, 4>;
-    if (v == NEOGEMM_VARIANT_SKINNY16) e = pick(I1{}, I4{}, I4{});
-    else if (v == NEOGEMM_VARIANT_SKINNY32) e = pick(I2{}, I3{}, I3{});
-    else if (v == NEOGEMM_VARIANT_SKINNY64) e = pick(I4{}, I2{}, I2{});
+    using I5 = integral_constant<int, 5>;
+    using I6 = integral_constant<int, 6>;
+    using I10 = integral_constant<int, 10>;
+    using W16 = integral_constant<int, 16>;
+    using W32 = integral_constant<int, 32>;
+    const int sw = sa.strip <= 16 ? 16 : sa.strip <= 32 ? 32 : 64;
+    if (v == NEOGEMM_VARIANT_SKINNY16) e = sw == 16 ? pick_narrow(I1{}, I10{}, W16{}) : sw == 32 ? pick_narrow(I1{}, I6{}, W32{}) : pick(I1{}, I4{}, I4{});
+    else if (v == NEOGEMM_VARIANT_SKINNY32) e = sw == 16 ? pick_narrow(I2{}, I6{}, W16{}) : sw == 32 ? pick_narrow(I2{}, I5{}, W32{}) : pick(I2{}, I3{}, I3{});
+    else if (v == NEOGEMM_VARIANT_SKINNY64) e = sw == 16 ? pick_narrow(I4{}, I4{}, W16{}) : sw == 32 ? pick_narrow(I4{}, I3{}, W32{}) : pick(I4{}, I2{}, I2{});
     // 65 to 128 rows, in sixteens: two steps of A and of B in the rings while they fit, else one of A and three of B
-    else if (sa.M <= 80) e = pick(integral_constant<int, 5>{}, I2{}, I2{});
-    else if (sa.M <= 96) e = pick(integral_constant<int, 6>{}, I2{}, I2{});
+    else if (sa.M <= 80) e = pick(I5{}, I2{}, I2{});
+    else if (sa.M <= 96) e = pick(I6{}, I2{}, I2{});
     else if (sa.M <= 112) e = pick(integral_constant<int, 7>{}, I3{}, I1{});
     else e = pick(integral_constant<int, 8>{}, I3{}, I1{});
     if (e != hipSuccess) {

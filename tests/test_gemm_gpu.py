@@ -740,7 +740,8 @@ def test_skinny_kernels(dev, variant, rows, b_layout, c_layout):
     # N: one strip, a ragged strip (N % 64, N % 8 == 0), many strips; M: 1, ragged, full
     for (M, N, K) in ((1, 64, 64), (rows, 200, 72), (rows - 3, 1000, 520), (rows - 4, 1000, 520), (rows, 4096, 1032),
                       (5, 2048, 8200), (8, 2048, 8200), (rows, 64, 4096), (3, 72, 136), (rows, 14336, 512),
-                      (rows // 2 + 1, 520, 1032), (rows // 2 + 4, 1096, 264), (rows - 16, 8, 256)):
+                      (rows // 2 + 1, 520, 1032), (rows // 2 + 4, 1096, 264), (rows - 16, 8, 256),
+                      (rows, 12280, 136)):   # B [N,K]: 256 strips of 48 columns, the last one 40 wide
         A, Bkn = o.make_inputs(M, N, K, seed=M + N + K)
         try:
             got = run_abi(A, layouts(Bkn, b_layout), dev, b_layout, c_layout, variant, strict=True)
@@ -749,6 +750,20 @@ def test_skinny_kernels(dev, variant, rows, b_layout, c_layout):
             assert e.status == _abi.ERR_UNSUPPORTED and c_layout == g.C_COL and M % 4 != 0
             continue
         o.assert_parity(got, A, Bkn, what=f"skinny v{variant} {M}x{N}x{K} b{b_layout} c{c_layout}")
+
+
+@pytest.mark.parametrize("variant,rows", SKINNY)
+def test_skinny_strip_widths_with_b_nk(dev, variant, rows):
+    """B [N,K]: the strips are as wide as fills the CUs in whole rounds (16 to 64 columns, multiples of 8; instances with
+    steps of 16, 32 and 64 columns); N need not be a multiple of 8 there, so the last strip can end anywhere."""
+    for (M, N, K) in ((rows, 4096, 264), (rows - 1, 6152, 200), (rows, 5004, 136), (3, 1004, 520), (rows, 8192, 72),
+                      (rows - 2, 14332, 136), (rows, 20480, 72), (rows, 24, 1032), (rows, 16388, 64)):
+        A, Bkn = o.make_inputs(M, N, K, seed=M + N + K)
+        for c_layout in (g.C_ROW, g.C_COL):
+            if c_layout == g.C_COL and M % 4 != 0:
+                continue   # ldc = M must be a multiple of 4 on the aligned path
+            got = run_abi(A, layouts(Bkn, g.B_NK), dev, g.B_NK, c_layout, variant, strict=True)
+            o.assert_parity(got, A, Bkn, what=f"skinny v{variant} {M}x{N}x{K} nk c{c_layout}")
 
 
 def test_skinny_known_answers_and_refusals(dev):
