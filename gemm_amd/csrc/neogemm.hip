@@ -1198,6 +1198,7 @@ struct SkinnyArgs {
   int M, N, K;
   long lda, ldb, ldc;
   float alpha, beta;
+  int rot;    // nonzero: workgroup b starts b * rot steps into its waves' shares of K and wraps around
   int strip;  // columns of C per workgroup: 64, or with B [N,K] a smaller multiple of 8 that fills the CUs better
 };
 // The end of the skinny kernels: the partial sums of the four waves (each over its share of K) meet in LDS (16 KiB * TMF
@@ -1304,7 +1305,20 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(SkinnyArgs p) {
   };
   // all loads of A / of B of step s of this wave into slot `slot` of that operand's ring; past K everything is
   // masked (the loads are still issued, as zero fills, so that the count of loads in flight does not depend on K)
-  auto issue_a = [&](int s, int slot) {
+  // Rows of a K-major B that lie a multiple of 16 KiB apart (K a multiple of 8192) and are all read at the same depth
+  // crowd onto a few memory channels: 16 x 14336 x 8192 runs 20 % faster, K = 16384 44 %, when every workgroup starts
+  // at another depth (other K: -3 .. +2 %, B [K,N]: -1 .. -5 %, so only there).  The order of a wave's sums then
+  // depends on the strip, not on anything that varies from run to run.
+  const int n_mine = s_end > s_begin ? (s_end - s_begin + s_stride - 1) / s_stride : 0;
+  const int rot0 = p.rot && n_mine > 0 ? (int)(blockIdx.x * p.rot) % n_mine : 0;
+  auto turn = [&](int s) {  // the step taken at the place of step s
+    if (!p.rot || s >= s_end) return s;
+    int i = (s - s_begin) / s_stride + rot0;
+    if (i >= n_mine) i -= n_mine;
+    return s_begin + i * s_stride;
+  };
+  auto issue_a = [&](int s0, int slot) {
+    const int s = turn(s0);
     const int krem = s < s_end ? p.K - s * KTILE : 0;  // depth left from this step on (<= 0: nothing)
     const uint32_t dst = ring_a + (uint32_t)slot * A_STEP;
     const i32x4 ra = rsrc((uint64_t)p.A + (uint64_t)s * KTILE * 2);
@@ -1317,7 +1331,8 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(SkinnyArgs p) {
       dma16<(j & 3) * 1024>(ra, v);
     });
   };
-  auto issue_b = [&](int s, int slot) {
+  auto issue_b = [&](int s0, int slot) {
+    const int s = turn(s0);
     const int krem = s < s_end ? p.K - s * KTILE : 0;
     const uint32_t dst = ring_b + (uint32_t)slot * B_STEP;
     const i32x4 rb = rsrc((uint64_t)p.B + (BKM ? ((uint64_t)n0 * p.ldb + (uint64_t)s * KTILE) * 2
@@ -1814,14 +1829,15 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
                   NEOGEMM_VARIANT_GENERIC, 1, 0, nullptr, alpha, beta, bt);
       return st2;
     }
-    SkinnyArgs sa{(const char*)A, (const char*)B, (char*)C, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, alpha, beta, 64};
+    SkinnyArgs sa{(const char*)A, (const char*)B, (char*)C, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, alpha, beta, 0, 64};
     bool bkm = b_layout == NEOGEMM_B_NK, ccol = c_layout == NEOGEMM_C_COL;
     if (swap) {
-      sa = SkinnyArgs{(const char*)B, (const char*)A, (char*)C, (int)N, (int)M, (int)K, (long)ldb, (long)lda, (long)ldc, alpha, beta, 64};
+      sa = SkinnyArgs{(const char*)B, (const char*)A, (char*)C, (int)N, (int)M, (int)K, (long)ldb, (long)lda, (long)ldc, alpha, beta, 0, 64};
       bkm = true;    // A [M,K] takes the place of a B [N,K]
       ccol = !ccol;  // a row-major C[m][n] is the column-major C^T
     }
     const bool wide = v == NEOGEMM_VARIANT_SKINNY128;
+    sa.rot = bkm && sa.ldb % 8192 == 0;  // rows of the wide operand a multiple of 16 KiB apart
     if (bkm) {
       // A strip of a K-major B may start at any row of it and be of any width that is a multiple of 8: the width is
       // chosen so that whole rounds of strips fill the CUs (N = 14336: 256 strips of 56 columns instead of 224 of 64,

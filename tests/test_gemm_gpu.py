@@ -757,7 +757,9 @@ def test_skinny_strip_widths_with_b_nk(dev, variant, rows):
     """B [N,K]: the strips are as wide as fills the CUs in whole rounds (16 to 64 columns, multiples of 8; instances with
     steps of 16, 32 and 64 columns); N need not be a multiple of 8 there, so the last strip can end anywhere."""
     for (M, N, K) in ((rows, 4096, 264), (rows - 1, 6152, 200), (rows, 5004, 136), (3, 1004, 520), (rows, 8192, 72),
-                      (rows - 2, 14332, 136), (rows, 20480, 72), (rows, 24, 1032), (rows, 16388, 64)):
+                      (rows - 2, 14332, 136), (rows, 20480, 72), (rows, 24, 1032), (rows, 16388, 64),
+                      # rows of B a multiple of 16 KiB apart: every strip starts at another depth of K
+                      (rows, 520, 8192), (rows - 1, 4100, 16384)):
         A, Bkn = o.make_inputs(M, N, K, seed=M + N + K)
         for c_layout in (g.C_ROW, g.C_COL):
             if c_layout == g.C_COL and M % 4 != 0:
