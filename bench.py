@@ -266,14 +266,29 @@ def main():
                 torch.matmul(ad, bds[it[0] % nbuf], out=c)
                 it[0] += 1
 
+            # the same with B stored [N,K], the reference's layout (neoGemmV1, nemgemmV03.cu:343-391)
+            bnks = [x.t().contiguous() for x in bds]
+
+            def fnk():
+                g.gemm_into(ad, bnks[it[0] % nbuf], c, m, n, k, k, k, n, g.B_NK, g.C_ROW)
+                it[0] += 1
+
+            def fvnk():
+                torch.matmul(ad, bnks[it[0] % nbuf].t(), out=c)
+                it[0] += 1
+
             ms = time_events(f, 200 if m * n * k < 2e11 else 50, 20)
             vms = time_events(fv, 200 if m * n * k < 2e11 else 50, 20)
+            ms_nk = time_events(fnk, 200 if m * n * k < 2e11 else 50, 20)
+            vms_nk = time_events(fvnk, 200 if m * n * k < 2e11 else 50, 20)
             fl, by = 2.0 * m * n * k, 2.0 * (m * k + k * n + m * n)
             v, s = g.plan(m, n, k)
             others.append({"M": m, "N": n, "K": k, "ms": round(ms, 5), "tflops": round(fl / ms / 1e9, 2),
                            "pct_of_2500": round(fl / ms / 1e9 / 25.0, 2), "gbps": round(by / ms / 1e6, 1),
                            "pct_of_8000": round(by / ms / 1e6 / 80.0, 2), "variant": g.VARIANT_NAMES[v], "split_k": s,
-                           "torch_matmul_ms": round(vms, 5)})
+                           "torch_matmul_ms": round(vms, 5), "ms_b_nk": round(ms_nk, 5),
+                           "variant_b_nk": g.VARIANT_NAMES[g.plan(m, n, k, g.B_NK, g.C_ROW)[0]],
+                           "torch_matmul_ms_b_nk": round(vms_nk, 5)})
         out["other_configs"] = others
 
     if args.calibrate_copy:
