@@ -1586,7 +1586,11 @@ static void plan_model(int64_t M, int64_t N, int64_t K, bool aligned, int c_layo
       const double lat_floor = __builtin_ceil(wgs / cus) * ktps * lat_us;
       if (t < lat_floor) t = lat_floor;
       t += rounds * (c.fixed_us + (sp > 1 ? c.split_fixed_us : 0.0));
-      if (t < stream_us) t = stream_us;
+      // fewer workgroups than CUs pull less from HBM: 112 of them 4.0 TB/s, 224 and more 5 and above (64x11008x14336
+      // with split 3, 129 workgroups: 87 us; split 4, 172: 73; 128x28672x14336 unsplit, 112: 230; split 2: 173)
+      const double fill = wgs < cus ? wgs / cus : 1.0;
+      const double floor_us = stream_us / (0.55 + 0.45 * fill);
+      if (t < floor_us) t = floor_us;
       if (sp > 1) t += 4.0 + (4.0 * sp + 2.0) * (double)rows * (double)cols * (double)batch / 5.0e6;
       if (t < best) {
         best = t;
