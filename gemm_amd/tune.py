@@ -22,7 +22,7 @@ from ._abi import B_KN, B_NK, C_COL, C_ROW, ERR_UNSUPPORTED, NeoGemmError
 
 CANDIDATE_VARIANTS = (_abi.VARIANT_T256x256_W4, _abi.VARIANT_C256x256_W4, _abi.VARIANT_T256x256_W8, _abi.VARIANT_T128x256_W4,
                       _abi.VARIANT_T256x128_W4, _abi.VARIANT_T128x128_W4, _abi.VARIANT_T64x128_W4,
-                      _abi.VARIANT_T192x256_W4, _abi.VARIANT_SKINNY16, _abi.VARIANT_SKINNY32, _abi.VARIANT_SKINNY64,
+                      _abi.VARIANT_T192x256_W4, _abi.VARIANT_T96x128_W4, _abi.VARIANT_T64x64_W4, _abi.VARIANT_SKINNY16, _abi.VARIANT_SKINNY32, _abi.VARIANT_SKINNY64,
                       _abi.VARIANT_SKINNY128)
 CANDIDATE_SPLITS = (1, 2, 3, 4, 6, 8, 12, 16, 24, 32)
 
