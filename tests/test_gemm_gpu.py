@@ -768,6 +768,40 @@ def test_skinny_strip_widths_with_b_nk(dev, variant, rows):
             o.assert_parity(got, A, Bkn, what=f"skinny v{variant} {M}x{N}x{K} nk c{c_layout}")
 
 
+def test_decode_shapes_through_the_plan_on_random_shapes(dev):
+    """Seeded random decode shapes (1 to 136 rows on either side, 2000 to 28672 columns, K from 520 to 14336), all
+    four layout pairs, through the auto plan: whatever kernel, strip width and ring the plan and the launcher pick, the
+    result meets the oracle's bar; small-integer data in the same shapes must come out exact."""
+    rng = np.random.default_rng(77)
+    seen = set()
+    for it in range(40):
+        small = int(rng.integers(1, 137))
+        wide = int(rng.choice([2048, 4096, 6144, 8192, 10240, 11008, 12288, 14336, 16384, 20480, 28672])) - 8 * int(rng.integers(0, 3))
+        K = int(rng.choice([520, 1024, 2048, 4096, 4104, 8192, 14336]))
+        if wide * K > 120e6:
+            wide = int(120e6 // K) // 8 * 8
+        tall = bool(rng.integers(0, 2))
+        M, N = (wide, small) if tall else (small, wide)
+        b_layout = g.B_NK if (tall or rng.integers(0, 2)) else g.B_KN
+        if b_layout == g.B_KN:
+            N = (N + 7) // 8 * 8          # whole 16-byte chunks of a row of B [K,N]
+        c_layout = g.C_COL if rng.integers(0, 2) else g.C_ROW
+        if (c_layout == g.C_COL and M % 4) or (c_layout == g.C_ROW and N % 4):
+            c_layout = g.C_ROW if N % 4 == 0 else g.C_COL
+        if (c_layout == g.C_COL and M % 4) or (c_layout == g.C_ROW and N % 4):
+            continue                      # neither leading dimension of C would be aligned
+        seen.add(g.plan(M, N, K, b_layout, c_layout)[0])
+        A, Bkn = o.make_inputs(M, N, K, seed=1000 + it)
+        got = run_abi(A, layouts(Bkn, b_layout), dev, b_layout, c_layout)
+        o.assert_parity(got, A, Bkn, what=f"decode {M}x{N}x{K} b{b_layout} c{c_layout}")
+        gen = torch.Generator().manual_seed(it)
+        Ai = torch.randint(-2, 3, (M, K), generator=gen).to(torch.bfloat16)
+        Bi = torch.randint(-2, 3, (K, N), generator=gen).to(torch.bfloat16)
+        goti = run_abi(Ai, layouts(Bi, b_layout), dev, b_layout, c_layout)
+        assert np.array_equal(o.bits_of(goti), o.bits_of(o.ref_gemm(Ai, Bi))), (M, N, K, b_layout, c_layout)
+    assert {g.VARIANT_SKINNY16, g.VARIANT_SKINNY64, g.VARIANT_SKINNY128} <= seen   # the draw reaches the decode kernels
+
+
 def test_skinny_known_answers_and_refusals(dev):
     gen = torch.Generator().manual_seed(31)
     for variant, rows in SKINNY:
