@@ -1172,13 +1172,14 @@ namespace neogemm {
 
 // ---------------------------------------------------------------------------------------------
 // Skinny M (decode shapes: M <= 16 * TMF; C row-major or, CCOL, column-major): bound by streaming B from HBM once, so what
-// counts is bytes in flight per CU, not MFMA rate.  A workgroup owns a strip of 64 columns of C and the
-// whole of K; no split-K, no second launch.  Its four waves split K between them in steps of 64,
+// counts is bytes in flight per CU, not MFMA rate.  A workgroup owns a strip of columns of C (64 with B [K,N]; with
+// B [N,K] as many, in eights up to 64, as fill the CUs in whole rounds: SkinnyArgs::strip, steps of SW = 16, 32 or 64
+// rows of B) and the whole of K; no split-K, no second launch.  Its four waves split K between them in steps of 64,
 // each with a private ring of RS steps in LDS that only it fills and reads:
 // no barrier until the end, when the four partial sums meet in LDS and are added in wave order.
 // One step of one wave: A 16*TMF rows x 128 B (K-major image, swz_k), B 64 k-rows x 128 B if B is [K,N]
-// (64 columns are one cache line per k-row; swizzle swz_mn64) or 64 rows x 128 B if B is [N,K].
-// 4 waves x (RA steps of A at 2 KiB * TMF + RS steps of B at 8 KiB) of LDS: TMF = 1 with rings of 4 fills the 160 KiB;
+// (64 columns are one cache line per k-row; swizzle swz_mn64) or SW rows x 128 B if B is [N,K].
+// 4 waves x (RA steps of A at 2 KiB * TMF + RS steps of B at SW * 128 B) of LDS, with SW = 64: TMF = 1 with rings of 4 fills the 160 KiB;
 // TMF = 2 with 3 and TMF = 4 with 2 (M <= 64: 30.5 us at 64x14336x4096, the split-K tile path 32.9) are the other
 // instances for up to 64 rows.  TMF = 5 .. 8 (up to 128 rows) fit two steps of each at most, or one of A and three of B.
 // A wave's loads complete in the order it issued them, so a ring deeper than the other operand's buys little: with one
