@@ -622,6 +622,23 @@ def run_scaled(A, B, C0, dev, alpha, beta, b_layout=g.B_KN, c_layout=g.C_ROW):
     return C if c_layout == g.C_ROW else C.t().contiguous()
 
 
+def test_scaled_through_the_decode_kernels(dev):
+    """alpha and beta through the skinny kernels the plan picks for decode shapes: 96 rows (SKINNY128), 16-column strips
+    (B [N,K], N = 4096) and staggered depths (K = 8192); exact on small integers, every layout of C."""
+    gen = torch.Generator().manual_seed(23)
+    for (M, N, K, b_layout, variant) in ((96, 14336, 2048, g.B_NK, g.VARIANT_SKINNY128), (96, 14336, 2048, g.B_KN, g.VARIANT_SKINNY128),
+                                         (16, 4096, 4096, g.B_NK, g.VARIANT_SKINNY16), (40, 8192, 8192, g.B_NK, g.VARIANT_SKINNY64)):
+        A = torch.randint(-2, 3, (M, K), generator=gen).to(torch.bfloat16)
+        B = torch.randint(-2, 3, (K, N), generator=gen).to(torch.bfloat16)
+        C0 = torch.randint(-8, 9, (M, N), generator=gen).to(torch.bfloat16)
+        for c_layout in (g.C_ROW, g.C_COL):
+            assert g.plan(M, N, K, b_layout, c_layout)[0] == variant
+            for alpha, beta in ((0.5, -3.0), (1.0, 1.0)):
+                want = o.ref_gemm_scaled(A, B, C0, alpha, beta)
+                got = run_scaled(A, layouts(B, b_layout), C0, dev, alpha, beta, b_layout, c_layout)
+                assert np.array_equal(o.bits_of(got), o.bits_of(want)), (M, N, K, alpha, beta, b_layout, c_layout)
+
+
 def test_scaled_exact_small_integers(dev):
     gen = torch.Generator().manual_seed(21)
     for (M, N, K) in ((24, 40, 16), (256, 512, 128), (130, 264, 72), (16, 2048, 1024)):   # generic, tile, ragged, split-K
