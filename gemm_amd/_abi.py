@@ -22,10 +22,11 @@ VARIANT_T192x256_W4 = 12
 VARIANT_T96x128_W4, VARIANT_T64x64_W4 = 13, 14
 VARIANT_C256x256_W4 = 15
 VARIANT_SKINNY128 = 16
-VARIANT_COUNT = 17
+VARIANT_STRIP = 17
+VARIANT_COUNT = 18
 VARIANT_NAMES = {0: "auto", 1: "generic", 2: "256x256_w8", 3: "256x256_w4", 4: "128x128_w4", 5: "256x128_w4",
                  6: "128x256_w4", 7: "64x128_w4", 8: "128x128_w4s", 9: "skinny16", 10: "skinny32", 11: "skinny64", 12: "192x256_w4", 13: "96x128_w4", 14: "64x64_w4",
-                 15: "256x256_w4_chain", 16: "skinny128"}
+                 15: "256x256_w4_chain", 16: "skinny128", 17: "strip"}
 
 # every symbol include/neogemm.h declares, with its prototype
 _i64, _int, _vp, _sz = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t

@@ -826,6 +826,20 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(TileArgs p) {
   }
 }
 
+// CUs of the current device (the runtime is asked once per device)
+inline hipError_t current_device_cus(int* out) {
+  static std::atomic<int> cus_of[64];
+  int dev = 0;
+  if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
+  int cus = dev >= 0 && dev < 64 ? cus_of[dev].load(std::memory_order_relaxed) : 0;
+  if (cus == 0) {
+    if (hipError_t e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev); e != hipSuccess) return e;
+    if (dev >= 0 && dev < 64) cus_of[dev].store(cus, std::memory_order_relaxed);
+  }
+  *out = cus;
+  return hipSuccess;
+}
+
 // Raise a kernel's dynamic-LDS limit once per (kernel, device): the attribute belongs to the current device's copy
 // of the function.  The registry is keyed on the kernel's address (all instances share one function-pointer type).
 template <class Kern>
@@ -866,7 +880,9 @@ hipError_t launch_tile(const TileArgs& a, bool ak, bool bk, hipStream_t st) {
   if (ak && bk) {
     if constexpr (BM == 128 && BN == 128) {
       // more workgroups than CUs: two images of B, 80 KiB, so that two workgroups share a CU
-      if ((int64_t)a.ntm * a.ntn * a.ksplit * a.batch > 256) {
+      int cus = 0;
+      if (hipError_t e = current_device_cus(&cus); e != hipSuccess) return e;
+      if ((int64_t)a.ntm * a.ntn * a.ksplit * a.batch > cus) {
         lds = (size_t)BM * 384 + (size_t)BN * 256;
         return go(gemm_tile_kernel<BM, BN, WGM, WGN, true, true, false, 2>);
       }
@@ -1081,20 +1097,6 @@ __global__ __launch_bounds__(256) void gemm_chain_kernel(TileArgs p) {
   else store_wave_tile<TM, TN, NW, LDS_BYTES>(acc, p, gC, kz, lane, wave, lds0, BlockMap{m0 + wm * 128, n0 + wn * 128});
 }
 
-// CUs of the current device (the runtime is asked once per device)
-inline hipError_t current_device_cus(int* out) {
-  static std::atomic<int> cus_of[64];
-  int dev = 0;
-  if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
-  int cus = dev >= 0 && dev < 64 ? cus_of[dev].load(std::memory_order_relaxed) : 0;
-  if (cus == 0) {
-    if (hipError_t e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev); e != hipSuccess) return e;
-    if (dev >= 0 && dev < 64) cus_of[dev].store(cus, std::memory_order_relaxed);
-  }
-  *out = cus;
-  return hipSuccess;
-}
-
 hipError_t launch_chain(const TileArgs& a, bool bk, hipStream_t st);
 #if NEOGEMM_HAS_PART(8)
 hipError_t launch_chain(const TileArgs& a, bool bk, hipStream_t st) {
@@ -1201,13 +1203,40 @@ struct SkinnyArgs {
   float alpha, beta;
   int rot;    // nonzero: workgroup b starts b * rot steps into its waves' shares of K and wraps around
   int strip;  // columns of C per workgroup: 64, or with B [N,K] a smaller multiple of 8 that fills the CUs better
+  int ra, rb; // gemm_strip_kernel: stages in the ring of A / of B
 };
+// One 16x16 fragment of sums (row fragment t, column fragment f of the strip at column n0) scaled and written to C.
+// The lane's four elements are consecutive along `fast` (n for a row-major C, m for a column-major one).
+template <bool CCOL>
+__device__ __forceinline__ void skinny_store_frag(f32x4 sum, int t, int f, const SkinnyArgs& p, int n0, int lane) {
+  const uint32_t frow = lane & 15, fq = (uint32_t)lane >> 4;
+  const int row = CCOL ? 16 * t + 4 * (int)fq : 16 * t + (int)frow;
+  const int col = CCOL ? n0 + 16 * f + (int)frow : n0 + 16 * f + 4 * (int)fq;
+  const int col_end = n0 + p.strip < p.N ? n0 + p.strip : p.N;  // a strip may be narrower than its fragments
+  if (row >= p.M || col >= col_end) return;
+  const int fast = CCOL ? row : col, fast_end = CCOL ? p.M : col_end;
+  char* cp = p.C + (CCOL ? (size_t)col * p.ldc + row : (size_t)row * p.ldc + col) * 2;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) sum[r] *= p.alpha;
+  if (p.beta != 0.f) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+      if (fast + r < fast_end) sum[r] = __builtin_fmaf(p.beta, (float)((const __bf16*)cp)[r], sum[r]);
+  }
+  const bf16x4 o = {(__bf16)sum[0], (__bf16)sum[1], (__bf16)sum[2], (__bf16)sum[3]};
+  if (fast + 3 < fast_end) {
+    *(bf16x4*)cp = o;
+  } else {
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+      if (fast + r < fast_end) ((__bf16*)cp)[r] = o[r];
+  }
+}
 // The end of the skinny kernels: the partial sums of the four waves (each over its share of K) meet in LDS (16 KiB * TMF
 // from `smem` on, which no wave may still be using) and wave w adds up fragment column w in wave order, scales and stores.
 template <int TMF, bool CCOL, int NF>
 __device__ __forceinline__ void skinny_reduce_store(f32x4 (&acc)[TMF][NF], const SkinnyArgs& p, int n0, int wave, int lane,
                                                     char* smem) {
-  const uint32_t frow = lane & 15, fq = (uint32_t)lane >> 4;
   NEOGEMM_AS3 f32x4* red = (NEOGEMM_AS3 f32x4*)smem;
 #pragma unroll
   for (int t = 0; t < TMF; ++t)
@@ -1224,28 +1253,7 @@ __device__ __forceinline__ void skinny_reduce_store(f32x4 (&acc)[TMF][NF], const
 #pragma unroll
       for (int r = 0; r < 4; ++r) sum[r] += v[r];
     }
-    // the lane's four elements are consecutive along `fast` (n for a row-major C, m for a column-major one)
-    const int row = CCOL ? 16 * t + 4 * (int)fq : 16 * t + (int)frow;
-    const int col = CCOL ? n0 + 16 * f + (int)frow : n0 + 16 * f + 4 * (int)fq;
-    const int col_end = n0 + p.strip < p.N ? n0 + p.strip : p.N;  // a strip may be narrower than its fragments
-    if (row >= p.M || col >= col_end) continue;
-    const int fast = CCOL ? row : col, fast_end = CCOL ? p.M : col_end;
-    char* cp = p.C + (CCOL ? (size_t)col * p.ldc + row : (size_t)row * p.ldc + col) * 2;
-#pragma unroll
-    for (int r = 0; r < 4; ++r) sum[r] *= p.alpha;
-    if (p.beta != 0.f) {
-#pragma unroll
-      for (int r = 0; r < 4; ++r)
-        if (fast + r < fast_end) sum[r] = __builtin_fmaf(p.beta, (float)((const __bf16*)cp)[r], sum[r]);
-    }
-    const bf16x4 o = {(__bf16)sum[0], (__bf16)sum[1], (__bf16)sum[2], (__bf16)sum[3]};
-    if (fast + 3 < fast_end) {
-      *(bf16x4*)cp = o;
-    } else {
-#pragma unroll
-      for (int r = 0; r < 4; ++r)
-        if (fast + r < fast_end) ((__bf16*)cp)[r] = o[r];
-    }
+    skinny_store_frag<CCOL>(sum, t, f, p, n0, lane);
   }
 }
 
@@ -1263,7 +1271,12 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(SkinnyArgs p) {
   const uint32_t lds0 = (uint32_t)(uintptr_t)(NEOGEMM_AS3 char*)smem;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int n0 = blockIdx.x * p.strip;
+  // workgroup -> strip: consecutive workgroup ids land on different XCDs; with a K-major wide operand id % 8 selects a
+  // contiguous run of strips (up to 1.5 % at K = 8192; with B [K,N], where neighbouring strips are neighbouring cache
+  // lines of every k-row, the plain order is 0.5 % ahead)
+  const int per = gridDim.x >> 3, rem = gridDim.x & 7, xcd = blockIdx.x & 7;
+  const int strip_id = BKM ? xcd * per + (xcd < rem ? xcd : rem) + (blockIdx.x >> 3) : (int)blockIdx.x;
+  const int n0 = strip_id * p.strip;
   const int nsteps = (p.K + KTILE - 1) / KTILE;
   const uint32_t ring_a = lds0 + (uint32_t)wave * WAVE_LDS, ring_b = ring_a + RA * A_STEP;
 
@@ -1311,7 +1324,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(SkinnyArgs p) {
   // at another depth (other K: -3 .. +2 %, B [K,N]: -1 .. -5 %, so only there).  The order of a wave's sums then
   // depends on the strip, not on anything that varies from run to run.
   const int n_mine = s_end > s_begin ? (s_end - s_begin + s_stride - 1) / s_stride : 0;
-  const int rot0 = p.rot && n_mine > 0 ? (int)(blockIdx.x * p.rot) % n_mine : 0;
+  const int rot0 = p.rot && n_mine > 0 ? (int)(strip_id * p.rot) % n_mine : 0;
   auto turn = [&](int s) {  // the step taken at the place of step s
     if (!p.rot || s >= s_end) return s;
     int i = (s - s_begin) / s_stride + rot0;
@@ -1420,6 +1433,211 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(SkinnyArgs p) {
   skinny_reduce_store<TMF, CCOL, NF>(acc, p, n0, wave, lane, smem);
 }
 
+// ---------------------------------------------------------------------------------------------
+// 65 to 128 rows again: the same strips, with rings that the waves share and eight waves to fill them.
+// What bounds these shapes is the path into the CU, not the matrix cores: every workgroup reads its strip of B once
+// from HBM and all of A from L2 (at 128 rows twice the bytes of its strip), and at 256 strips the L2s hand out A 256
+// times.  Requesting nothing but that, with no arithmetic at all, takes about 31 us at 128 x 14336 x 4096 with B [N,K]
+// (B alone: 22), however many requests are in flight; hipBLASLt runs the shape in 30.5.  gemm_skinny_kernel loses
+// another 3 us there for two reasons that this kernel removes: a wave gets one 1 KiB request accepted every ~56 cycles
+// while the CU's vector memory path takes one every ~20, so four waves that each request 24 KiB per step of 64 are
+// held up at issue; and the four partial sums of its K split meet in LDS at the end (128 KiB written, read back and
+// added while nothing else runs).
+// Here K is consumed in stages of 128 and a workgroup has eight waves.  Waves 0..3 compute: wave w owns a quarter of
+// the rows (whole 16-row fragments; TMF not a multiple of 4: the first TMF % 4 waves take one more, the others work on
+// their last one twice and drop the copy, so that the loop has no branches), all columns of the strip and all of K,
+// so there is nothing to add up at the end.  They also request B, a quarter of each stage per wave.  Waves 4..7
+// request A, a quarter of each stage per wave, and do nothing else.
+// One barrier per stage: behind it stage t has landed (each wave has waited for its own requests) and every wave is
+// past its reads of stage t - 1, whose slots are requested anew, R - 1 stages ahead, between the MFMAs of stage t.
+// LDS: [RA stages of A: two 64-deep K-major images of 16*TMF rows each][RB stages of B: two 64-deep images of 64 rows
+// (B [N,K]) or 128 k-rows of 64 columns (B [K,N])], laid out and swizzled as gemm_skinny_kernel's steps.
+// Stages past the end of K are requested as zero fills (resource size 0) so that the wait counts hold for every K.
+// Strips are handed out so that an XCD (workgroup id mod 8) owns a contiguous run of them, and with a K-major B every
+// strip starts at another stage of K and wraps around (see SkinnyArgs::rot).
+// ---------------------------------------------------------------------------------------------
+template <int N>
+__device__ __forceinline__ void wait_vmcnt_upto(int stages) {
+  // at most stages * N of this wave's loads may stay in flight (stages is wave-uniform; the count is an immediate)
+  switch (stages) {
+    case 0: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+    case 1: asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N <= 63 ? N : 63) : "memory"); break;
+    case 2: asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * N <= 63 ? 2 * N : 63) : "memory"); break;
+    case 3: asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * N <= 63 ? 3 * N : 63) : "memory"); break;
+    case 4: asm volatile("s_waitcnt vmcnt(%0)" ::"n"(4 * N <= 63 ? 4 * N : 63) : "memory"); break;
+    case 5: asm volatile("s_waitcnt vmcnt(%0)" ::"n"(5 * N <= 63 ? 5 * N : 63) : "memory"); break;
+    case 6: asm volatile("s_waitcnt vmcnt(%0)" ::"n"(6 * N <= 63 ? 6 * N : 63) : "memory"); break;
+    default: asm volatile("s_waitcnt vmcnt(%0)" ::"n"(7 * N <= 63 ? 7 * N : 63) : "memory"); break;
+  }
+}
+template <int TMF, bool BKM, bool CCOL>
+__global__ __launch_bounds__(512) void gemm_strip_kernel(SkinnyArgs p) {
+  static_assert(TMF >= 4 && TMF <= 8, "at least one row fragment per compute wave; 128 rows at most");
+  constexpr int NF = 4, STAGE_K = 128, RWF = (TMF + 3) / 4, NM = 4 * NF * RWF;  // row fragments, MFMAs per wave and stage
+  constexpr uint32_t A_SUB = TMF * 2048, A_STAGE = 2 * A_SUB, B_SUB = 8192, B_STAGE = 2 * B_SUB;
+  constexpr int NLA = TMF, NLB = 4;  // 1 KiB loads per stage of a wave that loads A / B: a quarter of the stage
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(NEOGEMM_AS3 char*)smem;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int quarter = wave & 3;  // the quarter of a stage of its operand this wave loads
+  // workgroup -> strip: consecutive workgroup ids land on different XCDs; id % 8 selects a contiguous run of strips
+  const int per = gridDim.x >> 3, rem = gridDim.x & 7, xcd = blockIdx.x & 7;
+  const int strip_id = xcd * per + (xcd < rem ? xcd : rem) + (blockIdx.x >> 3);
+  const int n0 = strip_id * p.strip;
+  const int nst = (p.K + STAGE_K - 1) / STAGE_K;
+  const int RA = p.ra, RB = p.rb;
+  const uint32_t ring_a = lds0, ring_b = lds0 + (uint32_t)RA * A_STAGE;
+  const int rot0 = p.rot ? (int)(((unsigned)strip_id * (unsigned)p.rot) % (unsigned)nst) : 0;
+
+  f32x4 acc[RWF][NF];
+#pragma unroll
+  for (int t = 0; t < RWF; ++t)
+#pragma unroll
+    for (int f = 0; f < NF; ++f)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) acc[t][f][v] = 0.f;
+  // a compute wave's row fragments are rf0 .. rf0 + nrf - 1
+  const int nrf = TMF / 4 + (quarter < TMF % 4 ? 1 : 0), rf0 = quarter * (TMF / 4) + (quarter < TMF % 4 ? quarter : TMF % 4);
+
+  auto run = [&](auto role) {
+    constexpr bool ROLE_A = decltype(role)::value;
+    constexpr bool KMAJ = ROLE_A || BKM;  // this wave's operand has K-contiguous rows
+    constexpr int NLOAD = ROLE_A ? NLA : NLB;
+    constexpr uint32_t STAGE = ROLE_A ? A_STAGE : B_STAGE, SUB = ROLE_A ? A_SUB : B_SUB;
+    const int R = ROLE_A ? RA : RB;
+    // A quarter of a stage.  K-major operand: half the rows (NLOAD * 8) of one 64-deep image; B [K,N]: 32 k-rows.
+    const int kq = KMAJ ? (quarter >> 1) * 64 : quarter * 32;  // depth of the quarter's first element within the stage
+    const int row0 = KMAJ ? (quarter & 1) * NLOAD * 8 : 0;    // its first row of the operand
+    const uint32_t ring = (ROLE_A ? ring_a : ring_b) + (KMAJ ? (uint32_t)(quarter >> 1) * SUB + (uint32_t)(quarter & 1) * NLOAD * 1024
+                                                             : (uint32_t)quarter * 4096);
+    // per-lane byte offsets of this wave's loads of a stage, relative to the first element of its quarter
+    // (instruction offsets and OOB_OFFSET as in Operand::init)
+    uint32_t vo[NLOAD];
+    const uint32_t ld = (uint32_t)(ROLE_A ? p.lda : p.ldb);
+#pragma unroll
+    for (int j = 0; j < NLOAD; ++j) {
+      const uint32_t r = 8 * j + (lane >> 3);  // row of the quarter (K-major) or its k-row (B [K,N])
+      const uint32_t c = (lane & 7) ^ (KMAJ ? swz_k(row0 + r) : swz_mn64(r));
+      vo[j] = r * ld * 2 + c * 16 + VOFF_BIAS - (j & 3) * 1024;
+      if constexpr (ROLE_A) {
+        if (row0 + (int)r >= p.M) vo[j] = OOB_OFFSET;
+      } else if constexpr (BKM) {
+        if (n0 + row0 + (int)r >= p.N || row0 + (int)r >= p.strip) vo[j] = OOB_OFFSET;  // rows past the strip: still issued, as zero fills
+      } else {
+        if (n0 + (int)c * 8 >= p.N || (int)c * 8 >= p.strip) vo[j] = OOB_OFFSET;
+      }
+    }
+    const uint64_t base0 = ROLE_A ? (uint64_t)p.A + ((uint64_t)row0 * p.lda + kq) * 2
+                           : BKM  ? (uint64_t)p.B + ((uint64_t)(n0 + row0) * p.ldb + kq) * 2
+                                  : (uint64_t)p.B + ((uint64_t)kq * p.ldb + n0) * 2;
+    const uint64_t kadv = KMAJ ? (uint64_t)STAGE_K * 2 : (uint64_t)STAGE_K * p.ldb * 2;
+    // all loads of this wave for stage s into the ring slot at `dst`: the first quarter of them at once, the others
+    // between the MFMAs of `mfmas` (none for a wave that only loads)
+    auto stage_loads = [&](int s, uint32_t dst, auto&& mfmas) {
+      const bool live = s < nst;
+      int ps = live ? s + rot0 : 0;
+      if (ps >= nst) ps -= nst;
+      // depth left from the quarter's first element on (K-major: < 64 is the K tail of its image; B [K,N]: < 32)
+      const int krem = live ? p.K - (ps * STAGE_K + kq) : 64;
+      const uint64_t b = base0 + (uint64_t)ps * kadv - VOFF_BIAS;
+      const i32x4 rs = {(int)(uint32_t)b, (int)(uint32_t)(b >> 32), live ? (int)0x80000000u : 0, 0x00020000};
+      constexpr int EARLY = (NLOAD + 3) / 4;
+      constexpr int NMF = ROLE_A ? 0 : NM;  // MFMAs of this wave per stage
+      static_for<NMF + 1>([&](auto mc) {
+        constexpr int m = decltype(mc)::value - 1;  // -1: ahead of the MFMAs
+        if constexpr (m >= 0) mfmas(std::integral_constant<int, (m >= 0 ? m : 0)>{});
+        static_for<NLOAD>([&](auto jc) {
+          constexpr int j = decltype(jc)::value;
+          if constexpr ((j < EARLY || NMF == 0 ? -1 : (j - EARLY) * NMF / (NLOAD - EARLY)) == m) {
+            uint32_t v = vo[j];
+            if (krem < 64) {
+              const uint32_t r = 8 * j + (lane >> 3);
+              if constexpr (KMAJ) {
+                const uint32_t c = (lane & 7) ^ swz_k(row0 + r);
+                if ((int)c * 8 >= krem) v = OOB_OFFSET;
+              } else {
+                if ((int)r >= krem) v = OOB_OFFSET;
+              }
+            }
+            if constexpr (j % 4 == 0) dma_set_m0(dst + (j / 4) * 4096);
+            dma16<(j & 3) * 1024>(rs, v);
+          }
+        });
+      });
+    };
+    // prologue: all but one stage of the ring
+    for (int s = 0; s < R - 1; ++s) stage_loads(s, ring + (uint32_t)s * STAGE, [](auto) {});
+    int slot_a = 0, slot_b = 0;  // slots of stage t in the two rings
+    int slot_ld = R - 1;         // slot of this wave's ring that takes the stage requested next
+    if constexpr (ROLE_A) {
+      for (int t = 0; t < nst; ++t) {
+        wait_vmcnt_upto<NLOAD>(R - 2);
+        __builtin_amdgcn_s_barrier();
+        stage_loads(t + R - 1, ring + (uint32_t)slot_ld * STAGE, [](auto) {});
+        slot_ld = slot_ld + 1 == R ? 0 : slot_ld + 1;
+      }
+    } else {
+      // fragment addresses within a stage (see FragReader and gemm_skinny_kernel): slab sl is the (sl & 1)-th half of the
+      // (sl >> 1)-th 64-deep image
+      const uint32_t frow = lane & 15, fq = (uint32_t)lane >> 4;
+      const uint32_t tr_r = frow >> 2, tr_c = frow & 3, kk = 8 * fq + tr_r;  // B [K,N]: k-row within the slab, the second read adds 4
+      auto k_off = [&](int sl) { return frow * 128 + (((4 * (uint32_t)(sl & 1) + fq) ^ swz_k(frow)) << 4); };
+      auto fa_off = [&](int sl) { return (uint32_t)(sl >> 1) * A_SUB + k_off(sl); };
+      auto fb_off = [&](int sl) { return BKM ? (uint32_t)(sl >> 1) * B_SUB + k_off(sl) : (32 * (uint32_t)sl + kk) * 128 + ((tr_c & 1) << 3); };
+      auto read_b = [&](uint32_t img_b, int f) -> bf16x8 {
+        if constexpr (BKM) {
+          return lds_read_b128(img_b + f * 2048);
+        } else {
+          const uint32_t ad = img_b + (((2 * f + (tr_c >> 1)) ^ swz_mn64(kk)) << 4);
+          const i16x4 lo = lds_read_tr16(ad), hi = lds_read_tr16(ad + 4 * 128);
+          return __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+        }
+      };
+      for (int t = 0; t < nst; ++t) {
+        // stage t has landed: this wave's requests for it (the R - 2 stages behind it may stay in flight), then everyone's;
+        // every wave is past its reads of stage t - 1, whose slot takes stage t + R - 1
+        wait_vmcnt_upto<NLOAD>(R - 2);
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        const uint32_t st_a = ring_a + (uint32_t)slot_a * A_STAGE, st_b = ring_b + (uint32_t)slot_b * B_STAGE;
+        bf16x8 af[4][RWF], bf[4][NF];
+#pragma unroll
+        for (int sl = 0; sl < 4; ++sl) {
+#pragma unroll
+          for (int f = 0; f < NF; ++f) bf[sl][f] = read_b(st_b + fb_off(sl), f);
+#pragma unroll
+          for (int i = 0; i < RWF; ++i) af[sl][i] = lds_read_b128(st_a + fa_off(sl) + (uint32_t)(rf0 + (i < nrf ? i : nrf - 1)) * 2048);
+        }
+        stage_loads(t + R - 1, ring + (uint32_t)slot_ld * STAGE, [&](auto mc) {
+          constexpr int m = decltype(mc)::value, sl = m / (NF * RWF), f = (m / RWF) % NF, i = m % RWF;
+          // B fragment first: a lane ends up with 4 consecutive n of one output row; for a column-major C the other way round
+          if constexpr (CCOL) acc[i][f] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[sl][i], bf[sl][f], acc[i][f], 0, 0, 0);
+          else acc[i][f] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bf[sl][f], af[sl][i], acc[i][f], 0, 0, 0);
+        });
+        // the fragments are in registers before this wave arrives at the next barrier, behind which their slots are rewritten
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        slot_a = slot_a + 1 == RA ? 0 : slot_a + 1;
+        slot_b = slot_b + 1 == RB ? 0 : slot_b + 1;
+        slot_ld = slot_ld + 1 == R ? 0 : slot_ld + 1;
+      }
+    }
+  };
+  if (wave >= 4) {
+    run(std::true_type{});
+    // the zero fills past the end of K have landed before the wave ends (nobody reads them)
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    return;
+  }
+  run(std::false_type{});
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+  for (int i = 0; i < RWF; ++i)
+#pragma unroll
+    for (int f = 0; f < NF; ++f)
+      if (i < nrf) skinny_store_frag<CCOL>(acc[i][f], rf0 + i, f, p, n0, lane);
+}
+
 // Sum the split-K partials in split order (deterministic) and round once to bf16.
 // Then C = alpha * sum + beta * C.
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ ws, char* C, int M, int N,
@@ -1512,6 +1730,7 @@ struct VariantInfo {
 static const VariantInfo kVariants[NEOGEMM_VARIANT_COUNT] = {
     {0, 0, 0}, {16, 16, 4}, {256, 256, 8}, {256, 256, 4}, {128, 128, 4}, {256, 128, 4}, {128, 256, 4}, {64, 128, 4}, {128, 128, 4},
     {16, 64, 4}, {32, 64, 4}, {64, 64, 4}, {192, 256, 4}, {96, 128, 4}, {64, 64, 4}, {256, 256, 4}, {128, 64, 4},
+    {128, 64, 4},
 };
 
 static bool is_aligned(const void* A, const void* B, const void* C, int64_t K, int64_t lda, int64_t ldb,
@@ -1543,8 +1762,21 @@ static const PlanCand kPlanCands[] = {
     {NEOGEMM_VARIANT_T64x128_W4, 0.35, 2.5, 1.0, 2},    {NEOGEMM_VARIANT_T192x256_W4, 1.04, 7.0, 9.0, 1},
     {NEOGEMM_VARIANT_T96x128_W4, 0.42, 2.8, 1.8, 1},    {NEOGEMM_VARIANT_T64x64_W4, 0.20, 2.0, 1.0, 2},
 };
+// CUs the model plans for: those of the current device, or 256 (one MI355X) where no device can be asked, as in a
+// host-only workspace query
+static int planning_cus() {
+  static std::atomic<bool> no_device{false};
+  if (no_device.load(std::memory_order_relaxed)) return 256;
+  int cus = 0;
+  if (current_device_cus(&cus) != hipSuccess || cus <= 0) {
+    (void)hipGetLastError();  // the failed query must not surface in a later call
+    no_device.store(true, std::memory_order_relaxed);
+    cus = 256;
+  }
+  return cus;
+}
 static void plan_model(int64_t M, int64_t N, int64_t K, bool aligned, int c_layout, int* variant, int* split_k,
-                       int64_t batch = 1, int b_layout = NEOGEMM_B_KN) {
+                       int64_t batch = 1, int b_layout = NEOGEMM_B_KN, int ncus = 256) {
   if (!aligned || K == 0) {
     *variant = NEOGEMM_VARIANT_GENERIC;
     *split_k = 1;
@@ -1552,7 +1784,7 @@ static void plan_model(int64_t M, int64_t N, int64_t K, bool aligned, int c_layo
   }
   const int64_t rows = c_layout == NEOGEMM_C_ROW ? M : N, cols = c_layout == NEOGEMM_C_ROW ? N : M;
   const int64_t ktiles = ceil_div(K, KTILE);
-  const double cus = 256.0;
+  const double cus = (double)ncus;
   const double bytes = 2.0 * ((double)rows * K + (double)K * cols + (double)rows * cols) * (double)batch;
   const double stream_us = bytes / 5.0e6, lat_us = bytes > 32e6 ? 0.7 : 0.3;
   static const int kSplits[] = {1, 2, 3, 4, 6, 8, 12, 16, 24, 32, 48, 64};
@@ -1632,23 +1864,36 @@ static void plan_model(int64_t M, int64_t N, int64_t K, bool aligned, int c_layo
       bs = 1;
     }
   }
-  // 65 to 128 rows (of M, or of N with B [N,K]): the same kernel with five to eight row fragments per wave.  Its rings
-  // hold two steps at most then, so it is only the better choice where one round of strips about fills the CUs and K
-  // is a few thousand deep (decode shapes like 128 x 14336 x 4096: 36.1 us against 39.5 for split-K tiles with B [N,K];
-  // with B [K,N] 39.4 against 36.9 at 128 rows, 37.5 against 41.2 at 112).  Fitted to such timings; the tile estimates
-  // above come out about an eighth below what those shapes measure, hence the factor.
+  // 65 to 128 rows (of M, or of N with B [N,K]): strips again, one launch, no workspace.  Up to 96 rows, and with
+  // B [K,N], gemm_skinny_kernel with five to eight row fragments per wave; its rings hold two steps at most then, so it
+  // is only the better choice where one round of strips about fills the CUs and K is a few thousand deep (with B [K,N]
+  // 39.4 us against 36.9 for split-K tiles at 128 x 14336 x 4096, 37.5 against 41.2 at 112 rows).  From 97 rows on with a
+  // K-major wide operand, gemm_strip_kernel (eight waves, shared rings, rows split between the waves): 4.7 us + the
+  // bytes a workgroup requests at 58 GB/s per round of strips (within 4 % of 100 and 128 rows x 8192 .. 28672 columns x
+  // 2048 .. 14336 deep; 128 x 14336 x 4096: 31.4 us against 34.0 for gemm_skinny_kernel, 18.2 against 20.8 at K = 2048).
+  // Fitted to such timings; the tile estimates above come out about an eighth below what those shapes measure, hence
+  // the factor.
   const bool wide_m = !skinny_m && !skinny_n && M <= 128;
   const bool wide_n = !skinny_m && !skinny_n && !wide_m && N <= 128 && b_layout == NEOGEMM_B_NK;
   if ((wide_m || wide_n) && batch == 1 && K >= 2048) {
     const int64_t rows = wide_m ? M : N, cols = wide_m ? N : M;
-    const double wgs = (double)ceil_div(cols, 64), full = __builtin_floor(wgs / cus), frac = wgs / cus - full;
+    const bool strip_kernel = b_layout == NEOGEMM_B_NK && rows > 96;
+    int w = 64;  // strip width: see launch_strip
+    if (strip_kernel) {
+      const int rounds = ceil_div(ceil_div(cols, 64), (int64_t)cus), ww = 8 * ceil_div(cols, 8 * (int64_t)rounds * (int64_t)cus);
+      if (ww >= 40 && ww < 64) w = ww;
+    }
+    const double wgs = (double)ceil_div(cols, w), full = __builtin_floor(wgs / cus), frac = wgs / cus - full;
     const double rounds = full + (frac > 0.0 ? 0.7 + 0.3 * frac : 0.0);
-    const double wg_bytes = (double)K * 128.0 + (double)ceil_div(rows, 16) * 16.0 * K * 2.0;
-    double t = 7.0 + rounds * wg_bytes / (b_layout == NEOGEMM_B_NK ? 52.0e3 : 46.0e3);
+    const double wg_bytes = (double)K * 2.0 * w + (double)ceil_div(rows, 16) * 16.0 * K * 2.0;
+    double t = strip_kernel ? 4.7 + rounds * wg_bytes / 58.0e3
+                            : 7.0 + rounds * wg_bytes / (b_layout == NEOGEMM_B_NK ? 52.0e3 : 46.0e3);
     if (t < stream_us) t = stream_us;
-    if (t < best * 1.12) {
+    // (with more than one round of strips the tile estimates are about right: 128 x 28672 x 4096 55 us for the tiles,
+    // 59.5 for the strips)
+    if (t < best * (strip_kernel && wgs > cus ? 1.0 : 1.12)) {
       best = t;
-      bv = NEOGEMM_VARIANT_SKINNY128;
+      bv = strip_kernel ? NEOGEMM_VARIANT_STRIP : NEOGEMM_VARIANT_SKINNY128;
       bs = 1;
     }
   }
@@ -1709,31 +1954,33 @@ static const std::vector<PlanEntry>& plan_table() {
   return table;
 }
 static void plan_uncached(int64_t M, int64_t N, int64_t K, bool aligned, int c_layout, int* variant, int* split_k,
-                          int64_t batch, int b_layout);
+                          int64_t batch, int b_layout, int ncus);
 // The cost model walks every (tile, split) candidate: a few microseconds on the host, as long as a small GEMM takes
 // on the GPU.  A caller in a loop repeats a handful of shapes, so each thread remembers its last few answers.
 static void plan(int64_t M, int64_t N, int64_t K, bool aligned, int c_layout, int* variant, int* split_k,
                  int64_t batch = 1, int b_layout = NEOGEMM_B_KN) {
   struct Memo {
     int64_t M = -1, N = -1, K = -1, batch = -1;
-    int b_layout = -1, c_layout = -1, aligned = -1, variant = 0, split_k = 0;
+    int b_layout = -1, c_layout = -1, aligned = -1, ncus = -1, variant = 0, split_k = 0;
   };
   static thread_local Memo memo[32];  // the workspace query alone asks for four layouts of a shape
   static thread_local unsigned next = 0;
+  const int ncus = planning_cus();
   for (const Memo& m : memo)
     if (m.M == M && m.N == N && m.K == K && m.batch == batch && m.b_layout == b_layout && m.c_layout == c_layout &&
-        m.aligned == (int)aligned) {
+        m.aligned == (int)aligned && m.ncus == ncus) {
       *variant = m.variant;
       *split_k = m.split_k;
       return;
     }
-  plan_uncached(M, N, K, aligned, c_layout, variant, split_k, batch, b_layout);
+  plan_uncached(M, N, K, aligned, c_layout, variant, split_k, batch, b_layout, ncus);
   Memo& m = memo[next++ & 31];
   m.M = M, m.N = N, m.K = K, m.batch = batch, m.b_layout = b_layout, m.c_layout = c_layout, m.aligned = (int)aligned;
+  m.ncus = ncus;
   m.variant = *variant, m.split_k = *split_k;
 }
 static void plan_uncached(int64_t M, int64_t N, int64_t K, bool aligned, int c_layout, int* variant, int* split_k,
-                          int64_t batch, int b_layout) {
+                          int64_t batch, int b_layout, int ncus) {
   if (aligned && K > 0 && batch == 1) {
     for (const PlanEntry& e : plan_table())
       if (e.M == M && e.N == N && e.K == K && e.c_layout == c_layout && e.b_layout == b_layout) {
@@ -1742,7 +1989,7 @@ static void plan_uncached(int64_t M, int64_t N, int64_t K, bool aligned, int c_l
         return;
       }
   }
-  plan_model(M, N, K, aligned, c_layout, variant, split_k, batch, b_layout);
+  plan_model(M, N, K, aligned, c_layout, variant, split_k, batch, b_layout, ncus);
 }
 
 // The largest split-K factor plan() returns for this shape over the four (b_layout, c_layout) combinations a call can
@@ -1757,6 +2004,62 @@ static int max_planned_split(int64_t M, int64_t N, int64_t K, int64_t batch) {
       if (s > best) best = s;
     }
   return best;
+}
+
+// Launch of gemm_strip_kernel (65 to 128 rows).  `rings` = 16 * RA + RB forces the ring depths (0: the defaults below).
+static int launch_strip(SkinnyArgs sa, bool bkm, bool ccol, int rings, hipStream_t st) {
+  int cus = 0;
+  if (hipError_t e = current_device_cus(&cus); e != hipSuccess) {
+    fprintf(stderr, "neogemm: device query failed: %s\n", hipGetErrorString(e));
+    return NEOGEMM_ERR_LAUNCH;
+  }
+  // Strips of 64 columns; of a K-major B (a strip is a set of whole rows then) the multiple of 8 from 40 up that fills
+  // the CUs in whole rounds (N = 14336: 256 strips of 56).  Strips of B [K,N] that are not 64 wide would share the cache
+  // lines at their edges with their neighbours: 128 x 14336 x 4096 takes 47 us with strips of 56 against 38 with 64.
+  sa.strip = 64;
+  if (bkm) {
+    const int rounds = ceil_div(ceil_div(sa.N, 64), cus), w = 8 * ceil_div(sa.N, 8 * (int64_t)rounds * cus);
+    if (w >= 40 && w < 64) sa.strip = w;
+    sa.rot = 1;  // every strip starts one stage further into K than the one before it: measured 3 to 5 % at K = 4096
+  }
+  const int tmf = ceil_div(sa.M, 16);
+  if (tmf < 5 || tmf > 8) return NEOGEMM_ERR_UNSUPPORTED;
+  // ring depths: three stages of A (4 KiB * tmf each: two in flight cover the way to L2 and back) and what the 160 KiB
+  // leave for B (16 KiB a stage)
+  static const int kRings[9][2] = {{0, 0}, {0, 0}, {0, 0}, {0, 0}, {0, 0}, {3, 6}, {3, 5}, {3, 4}, {3, 4}};
+  sa.ra = kRings[tmf][0];
+  sa.rb = kRings[tmf][1];
+  if (rings > 0) {
+    sa.ra = rings / 16;
+    sa.rb = rings % 16;
+  }
+  const size_t lds = (size_t)sa.ra * tmf * 4096 + (size_t)sa.rb * 16384;
+  // what the kernel assumes: a stage being read besides those in flight, wait counts within the counter's 6 bits,
+  // rings that fit the LDS
+  if (sa.ra < 2 || sa.rb < 2 || sa.ra > 9 || sa.rb > 9 || (sa.ra - 2) * tmf > 63 || (sa.rb - 2) * 4 > 63 || lds > 160 * 1024)
+    return NEOGEMM_ERR_UNSUPPORTED;
+  auto go = [&](auto kern) -> hipError_t {
+    if (hipError_t e = allow_lds(kern, lds); e != hipSuccess) return e;
+    kern<<<dim3(ceil_div(sa.N, sa.strip)), 512, lds, st>>>(sa);
+    return hipGetLastError();
+  };
+  auto pick = [&](auto tc) -> hipError_t {
+    constexpr int TMF = decltype(tc)::value;
+    if (bkm) return ccol ? go(gemm_strip_kernel<TMF, true, true>) : go(gemm_strip_kernel<TMF, true, false>);
+    return ccol ? go(gemm_strip_kernel<TMF, false, true>) : go(gemm_strip_kernel<TMF, false, false>);
+  };
+  hipError_t e = hipErrorInvalidValue;
+  switch (tmf) {
+    case 5: e = pick(std::integral_constant<int, 5>{}); break;
+    case 6: e = pick(std::integral_constant<int, 6>{}); break;
+    case 7: e = pick(std::integral_constant<int, 7>{}); break;
+    default: e = pick(std::integral_constant<int, 8>{}); break;
+  }
+  if (e != hipSuccess) {
+    fprintf(stderr, "neogemm: strip kernel launch failed: %s\n", hipGetErrorString(e));
+    return NEOGEMM_ERR_LAUNCH;
+  }
+  return NEOGEMM_OK;
 }
 
 // A batch of `count` problems of one shape; strides in elements between consecutive problems (0: shared operand).
@@ -1817,7 +2120,7 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
   if (!aligned) return NEOGEMM_ERR_UNSUPPORTED;
 
   if (v == NEOGEMM_VARIANT_SKINNY16 || v == NEOGEMM_VARIANT_SKINNY32 || v == NEOGEMM_VARIANT_SKINNY64 ||
-      v == NEOGEMM_VARIANT_SKINNY128) {
+      v == NEOGEMM_VARIANT_SKINNY128 || v == NEOGEMM_VARIANT_STRIP) {
     // what the skinny kernel assumes: M within its rows, whole 16-byte chunks of B [K,N] inside the matrix,
     // one problem.  If M is too large but N fits and B is [N,K], it runs the transposed problem
     // C^T = B * A^T: its small operand is B then, its wide one A, and the layout of C flips.
@@ -1843,6 +2146,7 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
     }
     const bool wide = v == NEOGEMM_VARIANT_SKINNY128;
     sa.rot = bkm && sa.ldb % 8192 == 0;  // rows of the wide operand a multiple of 16 KiB apart
+    if (v == NEOGEMM_VARIANT_STRIP) return launch_strip(sa, bkm, ccol, group_m, st);
     if (bkm) {
       // A strip of a K-major B may start at any row of it and be of any width that is a multiple of 8: the width is
       // chosen so that whole rounds of strips fill the CUs (N = 14336: 256 strips of 56 columns instead of 224 of 64,

@@ -68,9 +68,16 @@ extern "C" {
    K-major, K a multiple of 128, no split-K. */
 #define NEOGEMM_VARIANT_C256x256_W4 15
 /* M <= 128 by the same kernel (five to eight row fragments of 16 per wave, shorter rings): one launch, no workspace;
-   chosen where one round of strips about fills the CUs and K is a few thousand deep */
+   chosen for 65 to 96 rows (to 128 with B [K,N]) where one round of strips about fills the CUs and K is a few thousand deep */
 #define NEOGEMM_VARIANT_SKINNY128 16
-#define NEOGEMM_VARIANT_COUNT 17
+/* 65 <= M <= 128 (or, with B [N,K], 65 <= N <= 128 < M): strips of up to 64 columns and all of K per workgroup like
+   the skinny variants, but eight waves per workgroup and K in stages of 128 held in rings that the waves share: four
+   waves compute (a quarter of the rows each, so no partial sums meet at the end) and request B, four request A and do
+   nothing else.  One launch, no workspace; chosen from 97 rows on when the wide operand is K-major and one round of
+   strips about fills the CUs.  For this variant the group_m argument of neogemm_bf16_variant carries the ring depths,
+   16 * stages of A + stages of B (0: the defaults); rings that do not fit the 160 KiB of LDS are refused. */
+#define NEOGEMM_VARIANT_STRIP 17
+#define NEOGEMM_VARIANT_COUNT 18
 
 /*
  * C = A * op(B), bf16 in, fp32 accumulate, bf16 out.
@@ -158,8 +165,8 @@ int neogemm_bf16_variant(const void* A, const void* B, void* C, int64_t M, int64
  * `aligned` is nonzero when pointers and leading dimensions satisfy the MFMA path (16-byte / 8-element).
  * The choice comes from a cost model over the tile variants; if the environment variable
  * NEOGEMM_PLAN_TABLE names a JSON file of tuned choices (an array of objects with the integer fields
- * "M","N","K","c_layout","variant","split_k"; gemm_amd/tune.py writes one), an entry for the exact
- * shape wins.  The file is read once per process.
+ * "M","N","K","b_layout","c_layout","variant","split_k"; the layouts default to 0; gemm_amd/tune.py writes one), an
+ * entry for the exact shape and layouts wins.  The file is read once per process.
  */
 int neogemm_bf16_plan(int64_t M, int64_t N, int64_t K, int b_layout, int c_layout, int aligned,
                       int* variant, int* split_k);

@@ -77,13 +77,17 @@ def test_plan_for_the_benchmark_configs():
     assert _abi.plan(14336, 16, 4096, b_layout=_abi.B_KN)[0] not in (_abi.VARIANT_SKINNY16, _abi.VARIANT_GENERIC)
     # 65 to 128 rows with one round of strips over the CUs and a K of a few thousand: the streaming kernel in one launch
     # (measured: it beats split-K tiles there except at 128 rows with B [K,N]); elsewhere the tiles
-    for M in (65, 96, 128):
-        assert _abi.plan(M, 14336, 4096, b_layout=_abi.B_NK) == (_abi.VARIANT_SKINNY128, 1)
-        assert _abi.plan(14336, M, 4096, b_layout=_abi.B_NK, c_layout=_abi.C_COL) == (_abi.VARIANT_SKINNY128, 1)
+    # from 97 rows on with a K-major wide operand, the eight-wave strip kernel (shared rings, rows split between the waves)
+    for M, want in ((65, _abi.VARIANT_SKINNY128), (96, _abi.VARIANT_SKINNY128), (97, _abi.VARIANT_STRIP), (128, _abi.VARIANT_STRIP)):
+        assert _abi.plan(M, 14336, 4096, b_layout=_abi.B_NK) == (want, 1)
+        assert _abi.plan(14336, M, 4096, b_layout=_abi.B_NK, c_layout=_abi.C_COL) == (want, 1)
     assert _abi.plan(96, 14336, 4096, b_layout=_abi.B_KN) == (_abi.VARIANT_SKINNY128, 1)
-    assert _abi.plan(128, 14336, 4096, b_layout=_abi.B_KN)[0] != _abi.VARIANT_SKINNY128
-    for shape in ((128, 28672, 4096), (128, 4096, 14336), (128, 14336, 1024), (96, 6144, 4096), (129, 14336, 4096)):
-        assert _abi.plan(*shape, b_layout=_abi.B_NK)[0] != _abi.VARIANT_SKINNY128
+    assert _abi.plan(128, 14336, 4096, b_layout=_abi.B_KN)[0] not in (_abi.VARIANT_SKINNY128, _abi.VARIANT_STRIP)
+    assert _abi.plan(128, 8192, 2048, b_layout=_abi.B_NK) == (_abi.VARIANT_STRIP, 1)   # 14.8 us against 19.1 for split-K tiles
+    streaming = (_abi.VARIANT_SKINNY128, _abi.VARIANT_STRIP)
+    for shape in ((128, 28672, 4096), (128, 4096, 14336), (128, 14336, 1024), (96, 6144, 4096), (129, 14336, 4096),
+                  (128, 8192, 8192), (100, 4096, 4096)):
+        assert _abi.plan(*shape, b_layout=_abi.B_NK)[0] not in streaming
     # unaligned problems go to the generic kernel
     assert _abi.plan(100, 100, 100, aligned=False) == (_abi.VARIANT_GENERIC, 1)
     assert _abi.workspace_bytes(0, 5, 5) == 0 and _abi.workspace_bytes(5, 5, 0) == 0

@@ -623,10 +623,11 @@ def run_scaled(A, B, C0, dev, alpha, beta, b_layout=g.B_KN, c_layout=g.C_ROW):
 
 
 def test_scaled_through_the_decode_kernels(dev):
-    """alpha and beta through the skinny kernels the plan picks for decode shapes: 96 rows (SKINNY128), 16-column strips
+    """alpha and beta through the skinny kernels the plan picks for decode shapes: 96 rows (SKINNY128), 120 rows (STRIP), 16-column strips
     (B [N,K], N = 4096) and staggered depths (K = 8192); exact on small integers, every layout of C."""
     gen = torch.Generator().manual_seed(23)
     for (M, N, K, b_layout, variant) in ((96, 14336, 2048, g.B_NK, g.VARIANT_SKINNY128), (96, 14336, 2048, g.B_KN, g.VARIANT_SKINNY128),
+                                         (120, 14336, 2048, g.B_NK, g.VARIANT_STRIP),
                                          (16, 4096, 4096, g.B_NK, g.VARIANT_SKINNY16), (40, 8192, 8192, g.B_NK, g.VARIANT_SKINNY64)):
         A = torch.randint(-2, 3, (M, K), generator=gen).to(torch.bfloat16)
         B = torch.randint(-2, 3, (K, N), generator=gen).to(torch.bfloat16)
@@ -816,7 +817,7 @@ def test_decode_shapes_through_the_plan_on_random_shapes(dev):
         Bi = torch.randint(-2, 3, (K, N), generator=gen).to(torch.bfloat16)
         goti = run_abi(Ai, layouts(Bi, b_layout), dev, b_layout, c_layout)
         assert np.array_equal(o.bits_of(goti), o.bits_of(o.ref_gemm(Ai, Bi))), (M, N, K, b_layout, c_layout)
-    assert {g.VARIANT_SKINNY16, g.VARIANT_SKINNY64, g.VARIANT_SKINNY128} <= seen   # the draw reaches the decode kernels
+    assert {g.VARIANT_SKINNY16, g.VARIANT_SKINNY64, g.VARIANT_SKINNY128, g.VARIANT_STRIP} <= seen   # the draw reaches the decode kernels
 
 
 def test_skinny_known_answers_and_refusals(dev):
@@ -842,7 +843,8 @@ def test_skinny_known_answers_and_refusals(dev):
     # alpha/beta pass through
     assert g.plan(16, 14336, 4096)[0] == g.VARIANT_SKINNY16 and g.plan(64, 14336, 4096)[0] == g.VARIANT_SKINNY64
     assert g.plan(16, 14336, 4096, c_layout=g.C_COL)[0] == g.VARIANT_SKINNY16
-    assert g.plan(96, 14336, 4096)[0] == g.VARIANT_SKINNY128 and g.plan(128, 14336, 4096, b_layout=g.B_NK)[0] == g.VARIANT_SKINNY128
+    assert g.plan(96, 14336, 4096)[0] == g.VARIANT_SKINNY128 and g.plan(96, 14336, 4096, b_layout=g.B_NK)[0] == g.VARIANT_SKINNY128
+    assert g.plan(128, 14336, 4096, b_layout=g.B_NK)[0] == g.VARIANT_STRIP
     M, N, K = 16, 4096, 2048
     A, Bkn = o.make_inputs(M, N, K, seed=2)
     C0 = torch.randn(M, N, generator=gen).to(torch.bfloat16)
@@ -851,6 +853,89 @@ def test_skinny_known_answers_and_refusals(dev):
         got = run_scaled(A, Bkn, C0, dev, 1.5, -0.5, g.B_KN, c_layout)
         ulp, fro = o.scaled_parity(got, A, Bkn, C0, 1.5, -0.5)
         assert ulp <= 1.0 and fro <= 1e-3
+
+
+# ------------------------------------------------------------------------------------------------
+# 65 to 128 rows: the eight-wave strip kernel (shared rings, rows split between the compute waves), forced
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("b_layout", [g.B_KN, g.B_NK])
+@pytest.mark.parametrize("c_layout", [g.C_ROW, g.C_COL])
+def test_strip_kernel(dev, b_layout, c_layout):
+    # rows: every count of 16-row fragments from five to eight, whole and ragged (a wave then works on a copy of its last
+    # fragment and drops it); K: less than a stage, a partial stage, fewer stages than the rings hold, many, a K tail in
+    # the first and in the second half of a stage; N: one strip, ragged strips, two rounds of strips
+    for (M, N, K) in ((65, 64, 64), (80, 200, 72), (81, 1000, 520), (96, 1000, 392), (100, 4096, 1032), (112, 2048, 8200),
+                      (113, 64, 4096), (128, 72, 136), (128, 14336, 512), (127, 520, 1032), (124, 1096, 264), (68, 8, 256),
+                      (128, 12280, 136), (96, 28672, 256), (128, 3000, 2048 + 40), (72, 4104, 2048 + 104)):
+        if b_layout == g.B_KN and N % 8:
+            continue   # whole 16-byte chunks of a row of B [K,N]
+        A, Bkn = o.make_inputs(M, N, K, seed=M + N + K)
+        try:
+            got = run_abi(A, layouts(Bkn, b_layout), dev, b_layout, c_layout, g.VARIANT_STRIP, strict=True)
+        except g.NeoGemmError as e:
+            # a column-major C with ldc = M not a multiple of 4 is not on the aligned path: refused when forced
+            assert e.status == _abi.ERR_UNSUPPORTED and c_layout == g.C_COL and M % 4 != 0
+            continue
+        o.assert_parity(got, A, Bkn, what=f"strip {M}x{N}x{K} b{b_layout} c{c_layout}")
+
+
+def test_strip_kernel_known_answers_rings_and_refusals(dev):
+    gen = torch.Generator().manual_seed(37)
+    lib = _abi.load()
+    for (M, N, K) in ((128, 328, 200), (72, 64, 264), (97, 136, 1032), (112, 2048, 4096)):
+        A = torch.randint(-3, 4, (M, K), generator=gen).to(torch.bfloat16)
+        B = torch.randint(-3, 4, (K, N), generator=gen).to(torch.bfloat16)
+        want = o.ref_gemm(A, B)                                   # small integers: exact in any order
+        for b_layout in (g.B_KN, g.B_NK):
+            for c_layout in (g.C_ROW, g.C_COL):
+                if c_layout == g.C_COL and M % 4:
+                    continue
+                # the default rings and forced ones (the group_m argument carries 16 * stages of A + stages of B); rings
+                # that do not fit the 160 KiB of LDS, or with no stage in flight, are refused
+                for rings in (0, 0x22, 0x33, 0x25, 0x43, 0x99):
+                    Ad, Bd = A.to(dev), layouts(B, b_layout).to(dev)
+                    C = torch.full((M, N) if c_layout == g.C_ROW else (N, M), float("nan"), dtype=torch.bfloat16, device=dev)
+                    st = lib.neogemm_bf16_variant(Ad.data_ptr(), Bd.data_ptr(), C.data_ptr(), M, N, K, K, N if b_layout == g.B_KN else K,
+                                                  N if c_layout == g.C_ROW else M, b_layout, c_layout, None, 0, None,
+                                                  g.VARIANT_STRIP, 0, rings)
+                    tmf = (M + 15) // 16
+                    fits = rings == 0 or ((rings >> 4) * tmf * 4096 + (rings & 15) * 16384 <= 160 * 1024 and ((rings >> 4) - 2) * tmf <= 63)
+                    assert st == (_abi.OK if fits else _abi.ERR_UNSUPPORTED), (M, N, K, rings, st)
+                    if fits:
+                        torch.cuda.synchronize()
+                        got = C.cpu() if c_layout == g.C_ROW else C.cpu().t().contiguous()
+                        assert np.array_equal(o.bits_of(got), o.bits_of(want)), (M, N, K, b_layout, c_layout, rings)
+    # fewer than 65 or more than 128 rows on both sides, N % 8 != 0 with B [K,N]: refused, never mis-run
+    big = torch.zeros(129, 136, dtype=torch.bfloat16, device=dev)
+    call = lambda M_, N_, b_layout: lib.neogemm_bf16_variant(big.data_ptr(), big.data_ptr(), big.data_ptr(), M_, N_, 64, 64,
+                                                               136 if b_layout == 0 else 64, 136, b_layout, 0, None, 0, None, g.VARIANT_STRIP, 1, 0)
+    assert call(129, 136, 0) == _abi.ERR_UNSUPPORTED and call(64, 136, 0) == _abi.ERR_UNSUPPORTED
+    assert call(128, 132, 0) == _abi.ERR_UNSUPPORTED
+    assert call(129, 136, 1) == _abi.ERR_UNSUPPORTED   # B [N,K] with 136 rows: neither side has 65 to 128 rows
+    torch.cuda.synchronize()
+
+
+def test_strip_kernel_on_the_transposed_problem_and_through_the_plan(dev):
+    """N in 97 .. 128 < M with B [N,K] runs C^T = B * A^T on the strip kernel; the plan sends 97 to 128 rows with a K-major
+    wide operand there when one round of strips about fills the CUs."""
+    assert g.plan(128, 14336, 4096, b_layout=g.B_NK)[0] == g.VARIANT_STRIP
+    assert g.plan(14336, 112, 4096, b_layout=g.B_NK, c_layout=g.C_COL)[0] == g.VARIANT_STRIP
+    for (M, N, K) in ((14336, 128, 1024), (1000, 72, 520), (4100, 100, 2056), (14336, 112, 4096)):
+        A, Bkn = o.make_inputs(M, N, K, seed=M + N)
+        for c_layout in (g.C_ROW, g.C_COL):
+            if (c_layout == g.C_COL and M % 4) or (c_layout == g.C_ROW and N % 4):
+                continue
+            for v in (g.VARIANT_STRIP, None):
+                got = run_abi(A, layouts(Bkn, g.B_NK), dev, g.B_NK, c_layout, v, strict=True)
+                o.assert_parity(got, A, Bkn, what=f"strip-n v{v} {M}x{N}x{K} c{c_layout}")
+    # 128 x 14336 x 4096, the benchmark's decode shape, B [N,K], both layouts of C, bit-exact on small integers
+    gen = torch.Generator().manual_seed(41)
+    A = torch.randint(-2, 3, (128, 4096), generator=gen).to(torch.bfloat16)
+    B = torch.randint(-2, 3, (4096, 14336), generator=gen).to(torch.bfloat16)
+    want = o.ref_gemm(A, B)
+    for c_layout in (g.C_ROW, g.C_COL):
+        got = run_abi(A, layouts(B, g.B_NK), dev, g.B_NK, c_layout)
+        assert np.array_equal(o.bits_of(got), o.bits_of(want))
 
 
 def test_narrow_operands_run_the_tile_kernels(dev):
