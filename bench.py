@@ -5,9 +5,12 @@
 
 Prints ONE JSON line.  A step is one GEMM (A [M,K] @ B [K,N], bf16 in, fp32 accumulate, bf16 out) on
 inputs already resident in HBM.  Order of events:
+  0. a host thread starts polling the board's telemetry (socket power, shader clocks: gemm_amd/telemetry.py, amdsmi;
+     no GPU call, no process) and keeps doing so to the end: `roofline.power` holds what it read during each leg;
   1. (before this process touches the GPU) the stand-alone harness gemm_amd/vendor_bench/matmul_bench runs as a
      child: the matrix cores' power ceiling on N(0,1) operands (`roofline.power_ceiling`), and hipBLASLt (best of
-     its heuristic candidates) / rocBLAS / libneogemm on the same buffers, both layouts of B (`vendor`);
+     its heuristic candidates) / rocBLAS / libneogemm on the same buffers, both layouts of B (`vendor`); with --all
+     also the other benchmark configurations, the same way (`other_configs`);
   2. an untimed, time-based preheat of the very GEMM that is measured (`preheat_ms`): the chip is power-limited
      on random data and the first launches after an idle period run slower until the clocks have settled;
   3. W warm-up steps, then exactly K timed steps between two synchronisations: `value` = 2*M*N*K / wall time per
@@ -15,7 +18,8 @@ inputs already resident in HBM.  Order of events:
      is `roofline.kernel_ms`, the list is `roofline.batch_ms`;
   4. parity spot check against the CPU oracle, and the oracle's own fp32 product timed on the host cores
      (`cpu_baseline`: a reported baseline, not a target).
-With --all the other benchmark configurations are timed too and reported under `other_configs`.
+`roofline.frac_of_power_ceiling` divides by the ceiling of the MFMA order the timed kernel issues
+(`roofline.power_ceiling_order`), measured in this run.
 """
 import argparse
 import json
@@ -53,7 +57,7 @@ def run_harness(args, env_extra=None, timeout=300):
     return rows
 
 
-def vendor_leg(M, N, K, preheat_ms):
+def vendor_leg(M, N, K, preheat_ms, sampler=None):
     """hipBLASLt best-of-heuristics, rocBLAS and libneogemm timed by one harness on the same buffers, B [K,N] and [N,K]."""
     out = {"harness": "gemm_amd/vendor_bench/matmul_bench (child process, HIP events, median of 5 batches of 40, "
                       f"{preheat_ms} ms preheat per library)"}
@@ -64,15 +68,67 @@ def vendor_leg(M, N, K, preheat_ms):
                 out[f"{r['lib']}_tflops_{name}"] = r["tflops"]
                 if r["lib"] == "hipblaslt":
                     out[f"hipblaslt_algos_tried_{name}"] = r.get("algos_tried")
+                if sampler is not None and "t0" in r:
+                    out.setdefault("power", {})[f"{r['lib']}_{name}"] = brief(sampler.summary(r["t0"], r["t1"]))
             elif r.get("check") == "neogemm_vs_vendor":
                 out[f"rel_fro_vs_vendor_{name}"] = r["rel_fro"]
     return out
 
 
-def power_ceiling(preheat_ms):
+def brief(summary):
+    """mean socket power and shader clock of a telemetry summary, for the per-leg tables"""
+    if not summary.get("available") or not summary.get("samples"):
+        return None
+    return {"socket_power_w": summary.get("socket_power_w", {}).get("mean"),
+            "shader_clock_mhz": summary.get("shader_clock_mhz", {}).get("mean"), "samples": summary["samples"]}
+
+
+# the other benchmark configurations: (M, N, K, weight buffers to rotate through, repetitions per batch)
+OTHER_CONFIGS = ((512, 512, 512, 1, 200), (4096, 4096, 4096, 1, 40), (16, 14336, 4096, 8, 100), (64, 14336, 4096, 8, 100),
+                 (128, 14336, 4096, 8, 100), (3000, 5120, 3584, 1, 40), (1024, 1024, 32768, 1, 40))
+
+
+def other_configs_leg(preheat_ms, sampler=None):
+    """Every other benchmark configuration the way the headline's vendor leg is measured: one child per shape and layout
+    of B, libneogemm / hipBLASLt best of its heuristic candidates / rocBLAS on the same buffers, a time-based preheat of
+    each library before it is timed, weights of the decode shapes rotating through 8 buffers (940 MB)."""
+    rows_out = []
+    for (m, n, k, nbuf, reps) in OTHER_CONFIGS:
+        fl, by = 2.0 * m * n * k, 2.0 * (m * k + k * n + m * n)
+        row = {"M": m, "N": n, "K": k, "weight_buffers": nbuf}
+        for bl, name in ((0, "b_kn"), (1, "b_nk")):
+            for r in run_harness([m, n, k, reps, bl, 0, 0, 0, nbuf], {"MATMUL_BENCH_PREHEAT_MS": str(preheat_ms)}):
+                if "lib" not in r:
+                    continue
+                us = r["ms"] * 1e3
+                if r["lib"] == "neogemm":
+                    row[f"us_{name}"] = round(us, 2)
+                    row[f"tflops_{name}"] = round(fl / us / 1e6, 2)
+                    row[f"pct_of_2500_{name}"] = round(fl / us / 1e6 / 25.0, 2)
+                    row[f"gbps_{name}"] = round(by / us / 1e3, 1)
+                    row[f"pct_of_8000_{name}"] = round(by / us / 1e3 / 80.0, 2)
+                    row[f"variant_{name}"], row[f"split_k_{name}"] = r.get("variant"), r.get("split_k")
+                    if sampler is not None and "t0" in r:
+                        row[f"power_{name}"] = brief(sampler.summary(r["t0"], r["t1"]))
+                else:
+                    row[f"{r['lib']}_us_{name}"] = round(us, 2)
+        rows_out.append(row)
+    return rows_out
+
+
+def power_ceiling(preheat_ms, sampler=None):
     rows = [r for r in run_harness(["ceiling", preheat_ms]) if "ceiling" in r]
     if not rows:
         return None
+    if sampler is not None:
+        # what the board's telemetry read while each MFMA-only case was being timed
+        tele = {}
+        for r in rows:
+            if "t0" not in r or r["ceiling"] == "gemm_like":
+                continue
+            key = (r.get("order") or ("16x16x32" if "16x16x32" in r["ceiling"] else "32x32x16")) + ", " + r["operands"]
+            tele[key] = brief(sampler.summary(r["t0"], r["t1"]))
+        power_ceiling.telemetry = tele
     out = {"what": "MFMA-only loop from registers, one wave per SIMD on 256 CUs, measured in this run before the GEMM "
                    "(matmul_bench ceiling): the rate the chip's power limit allows the matrix cores alone",
            "unit": "TFLOP/s"}
@@ -122,10 +178,15 @@ def main():
     M = N = K = 8192
 
     # child runs first: this process has not initialised the GPU yet
-    ceiling = vendor = None
+    from gemm_amd.telemetry import Sampler   # imports neither torch nor HIP
+    sampler = Sampler().start()
+    ceiling = vendor = others = None
+    power_ceiling.telemetry = {}
     if not args.no_vendor:
-        ceiling = power_ceiling(700)
-        vendor = vendor_leg(M, N, K, 1000)
+        ceiling = power_ceiling(700, sampler)
+        vendor = vendor_leg(M, N, K, 1000, sampler)
+        if args.all:
+            others = other_configs_leg(300, sampler)
 
     import torch
 
@@ -150,6 +211,7 @@ def main():
             raise g.NeoGemmError(st)
 
     # 2. preheat (time-based, untimed)
+    mono_pre = time.monotonic()
     t_pre = time.perf_counter()
     while (time.perf_counter() - t_pre) * 1e3 < args.preheat_ms:
         for _ in range(20):
@@ -163,6 +225,7 @@ def main():
     sizes = [args.steps // nb + (1 if i < args.steps % nb else 0) for i in range(nb)]
     ev = [torch.cuda.Event(enable_timing=True) for _ in range(nb + 1)]
     torch.cuda.synchronize()
+    mono_t0 = time.monotonic()
     t0 = time.perf_counter()
     ev[0].record(stream)
     for i, n in enumerate(sizes):
@@ -171,6 +234,7 @@ def main():
         ev[i + 1].record(stream)
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    mono_t1 = time.monotonic()
     batch_ms = [ev[i].elapsed_time(ev[i + 1]) / sizes[i] for i in range(nb)]
     kernel_ms = sorted(batch_ms)[nb // 2]
     flop = 2.0 * M * N * K
@@ -195,10 +259,22 @@ def main():
                 "traffic": measured_traffic(),
                 "kernel_ms": round(kernel_ms, 5), "batch_ms": [round(b, 5) for b in batch_ms],
                 "flop_per_launch": flop, "algorithmic_bytes": 2.0 * (M * K + K * N + M * N)}
+    # what the board itself reported while the timed kernel ran (and, for comparison, during the MFMA-only ceiling runs)
+    roofline["power"] = {"timed_region": sampler.summary(mono_t0, mono_t1),
+                         "preheat_and_timed": brief(sampler.summary(mono_pre, mono_t1)),
+                         "mfma_only_ceiling_runs": power_ceiling.telemetry or None}
     if ceiling:
         roofline["power_ceiling"] = ceiling
+        # the ceiling of the MFMA order the timed kernel issues: the chained kernel accumulates twice in a row into each
+        # tile, the slab kernel walks 2x2 blocks of tiles
+        order = ("2x2 blocks, both K steps of a tile back to back" if variant == g.VARIANT_C256x256_W4
+                 else "2x2 blocks, serpentine")
+        by_order = ceiling.get("by_mfma_order_randn", {})
+        if by_order.get(order):
+            roofline["power_ceiling_order"] = order
+            roofline["frac_of_power_ceiling"] = round(achieved / by_order[order], 4)
         if ceiling.get("16x16x32_randn"):
-            roofline["frac_of_power_ceiling"] = round(achieved / ceiling["16x16x32_randn"], 4)
+            roofline["frac_of_plain_order_ceiling"] = round(achieved / ceiling["16x16x32_randn"], 4)
 
     out = {
         "metric": "BF16 GEMM TFLOP/s at 8192^3 on 1 MI355X; % of dense-BF16 peak",
@@ -248,48 +324,11 @@ def main():
         "neogemm_tflops_b_nk": round(flop / time_events(
             lambda: g.gemm_into(Ad, Bnk, C, M, N, K, K, K, N, g.B_NK, g.C_ROW), n_t, 10) / 1e9, 2)}
 
-    if args.all:
-        others = []
-        for (m, n, k) in ((512, 512, 512), (4096, 4096, 4096), (16, 14336, 4096), (64, 14336, 4096),
-                          (128, 14336, 4096), (3000, 5120, 3584), (1024, 1024, 32768)):
-            a, b = o.make_inputs(m, n, k, seed=1)
-            nbuf = 8 if m <= 128 else 1   # rotate weights larger than the 256 MB last-level cache
-            ad, bds = a.to(dev), [b.to(dev).clone() for _ in range(nbuf)]
-            c = torch.empty(m, n, dtype=torch.bfloat16, device=dev)
-            it = [0]
-
-            def f():
-                g.gemm_into(ad, bds[it[0] % nbuf], c, m, n, k, k, n, n, g.B_KN, g.C_ROW)
-                it[0] += 1
-
-            def fv():
-                torch.matmul(ad, bds[it[0] % nbuf], out=c)
-                it[0] += 1
-
-            # the same with B stored [N,K], the reference's layout (neoGemmV1, nemgemmV03.cu:343-391)
-            bnks = [x.t().contiguous() for x in bds]
-
-            def fnk():
-                g.gemm_into(ad, bnks[it[0] % nbuf], c, m, n, k, k, k, n, g.B_NK, g.C_ROW)
-                it[0] += 1
-
-            def fvnk():
-                torch.matmul(ad, bnks[it[0] % nbuf].t(), out=c)
-                it[0] += 1
-
-            ms = time_events(f, 200 if m * n * k < 2e11 else 50, 20)
-            vms = time_events(fv, 200 if m * n * k < 2e11 else 50, 20)
-            ms_nk = time_events(fnk, 200 if m * n * k < 2e11 else 50, 20)
-            vms_nk = time_events(fvnk, 200 if m * n * k < 2e11 else 50, 20)
-            fl, by = 2.0 * m * n * k, 2.0 * (m * k + k * n + m * n)
-            v, s = g.plan(m, n, k)
-            others.append({"M": m, "N": n, "K": k, "ms": round(ms, 5), "tflops": round(fl / ms / 1e9, 2),
-                           "pct_of_2500": round(fl / ms / 1e9 / 25.0, 2), "gbps": round(by / ms / 1e6, 1),
-                           "pct_of_8000": round(by / ms / 1e6 / 80.0, 2), "variant": g.VARIANT_NAMES[v], "split_k": s,
-                           "torch_matmul_ms": round(vms, 5), "ms_b_nk": round(ms_nk, 5),
-                           "variant_b_nk": g.VARIANT_NAMES[g.plan(m, n, k, g.B_NK, g.C_ROW)[0]],
-                           "torch_matmul_ms_b_nk": round(vms_nk, 5)})
-        out["other_configs"] = others
+    if others is not None:
+        out["other_configs"] = {"method": "gemm_amd/vendor_bench/matmul_bench, one child per shape and layout of B, run before this "
+                                          "process touched the GPU: 300 ms preheat per library, median of 5 event-timed batches; "
+                                          "hipBLASLt = best of 8 heuristic candidates; columns *_b_kn: B [K,N], *_b_nk: B [N,K]",
+                                "rows": others}
 
     if args.calibrate_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
@@ -313,6 +352,7 @@ def main():
                                "sample": f"full M=N=K=8192 fp32 torch.matmul on the host, median of 5 ({dt:.1f} s each), "
                                          f"{os.cpu_count()} logical CPUs visible",
                                "seconds": round(dt, 2)}
+    sampler.stop()
     print(json.dumps(out), flush=True)
 
 

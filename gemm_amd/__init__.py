@@ -18,7 +18,8 @@ from ._abi import (B_KN, B_NK, C_COL, C_ROW, NeoGemmError, VARIANT_AUTO, VARIANT
 
 __all__ = ["gemm", "neoGemmV1", "neogemm", "gemm_into", "plan", "workspace_bytes", "version", "NeoGemmError"]
 
-_workspaces = {}
+_workspaces = {}        # (device index, stream) -> buffer, in order of last use
+_MAX_WORKSPACES = 16    # streams come and go: the least recently used buffer is dropped beyond this many
 
 
 def _check(t, name):
@@ -35,16 +36,18 @@ def _check(t, name):
 def _workspace(device, nbytes):
     """Split-K scratch for torch's current stream on `device`: one buffer per (device, stream), so that GEMMs on
     different streams never share partials.  A buffer is allocated while its stream is current and used on that
-    stream only, so when a larger one replaces it the caching allocator reuses the block in that stream's order."""
+    stream only, so when a larger one replaces it, or it is dropped as the least recently used of too many, the
+    caching allocator reuses the block in that stream's order."""
     with torch.cuda.device(device):
         key = (device.index if device.index is not None else torch.cuda.current_device(),
                torch.cuda.current_stream().cuda_stream)
-        ws = _workspaces.get(key)
+        ws = _workspaces.pop(key, None)
         if ws is None or ws.numel() < nbytes:
-            _workspaces.pop(key, None)
             ws = None
+            while len(_workspaces) >= _MAX_WORKSPACES:
+                _workspaces.pop(next(iter(_workspaces)))
             ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
-            _workspaces[key] = ws
+        _workspaces[key] = ws   # (re)inserted last: dicts keep insertion order
     return ws
 
 

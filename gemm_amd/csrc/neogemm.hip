@@ -336,11 +336,6 @@ struct BlockMap {  // one block
   __device__ __forceinline__ int row(int l) const { return r0 + l; }
   __device__ __forceinline__ int col(int l) const { return c0 + l; }
 };
-struct QuadMap {  // local 64-row / 64-column halves lie 128 apart (gemm_chain_kernel)
-  int r0, c0;
-  __device__ __forceinline__ int row(int l) const { return r0 + ((l >> 6) << 7) + (l & 63); }
-  __device__ __forceinline__ int col(int l) const { return c0 + ((l >> 6) << 7) + (l & 63); }
-};
 
 // Epilogue of the tile kernels: the TM x TN accumulator tiles of a wave (NW waves per workgroup, LDS_BYTES of LDS
 // that the main loop is done with) go to C as bf16, or to the split-K partials as fp32.
@@ -912,9 +907,10 @@ hipError_t launch_tile(const TileArgs& a, bool ak, bool bk, hipStream_t st) {
 //                a block (2 columns x 2 rows x 2 steps) goes (c0,i0,k0) (c0,i0,k1) (c0,i1,k0) (c0,i1,k1) (c1,i1,k0) ...
 // LDS: A two 64-deep tile images (32 KiB each), B three (K-major: a tile image; MN-major: two 32-deep slab images),
 // laid out and swizzled as in gemm_tile_kernel.  During period q a wave loads A tile q+2 over tile q (whose fragments
-// it read during the second half of period q-1) and B tile q+2 over tile q-1: all sixteen loads in the first half.
-// Two barriers per period: at its start (everyone is done reading what the period's loads overwrite) and in the
-// middle (A tile q+1 and B tile q+1, requested during period q-1, have landed: they are read during the second half).
+// it read during the last third of period q-1) and B tile q+2 over tile q-1: one load behind every seventh MFMA, the
+// last of the sixteen behind MFMA 107 of 128.
+// Two barriers per period: at its start (everyone is done reading what the period's loads overwrite) and before MFMA 88
+// (A tile q+1 and B tile q+1, requested during period q-1, have landed: they are read during the rest of the period).
 // K is a multiple of 128 and not split; a tile past the end of K is requested all the same, as a zero fill.
 // ---------------------------------------------------------------------------------------------
 template <bool BK>
@@ -926,14 +922,8 @@ __global__ __launch_bounds__(256) void gemm_chain_kernel(TileArgs p) {
   constexpr int IA = OpA::IPW, IB = OpB::IPW;          // loads of this wave per unit (A: a tile; B: a tile or a slab)
   constexpr int UB = KTILE / OpB::UNIT_K, LB = IB * UB;  // B units, B loads per period
   static_assert(IA == 8 && LB == 8, "eight loads per operand, wave and period");
-#ifndef PAIR_LANDED_AT
-#define PAIR_LANDED_AT 88
-#endif
-#ifndef PAIR_LOAD_STEP
-#define PAIR_LOAD_STEP 7
-#endif
-  constexpr int LOAD_STEP = PAIR_LOAD_STEP;  // a load behind every LOAD_STEP-th MFMA from the third on
-  constexpr int LANDED_AT = PAIR_LANDED_AT;  // MFMA of the period before which the barrier for tile q+1 sits (even, 64..96)
+  constexpr int LOAD_STEP = 7;   // a load behind every LOAD_STEP-th MFMA from the third on: the sixteenth behind MFMA 107
+  constexpr int LANDED_AT = 88;  // MFMA of the period before which the barrier for tile q+1 sits (even, 64..96); both tuned on the GPU
 
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   const uint32_t lds0 = (uint32_t)(uintptr_t)(NEOGEMM_AS3 char*)smem;
@@ -1062,13 +1052,13 @@ __global__ __launch_bounds__(256) void gemm_chain_kernel(TileArgs p) {
           fb[nb][cc][kk] = with_half(fb[nb][cc][kk], lds_read_tr16(a), h);
         }
       }
-      // A: the next tile's sixteen fragments behind the even MFMAs 64..94 (B's reads sit behind odd ones); done well
+      // A: the next tile's sixteen fragments behind the even MFMAs LANDED_AT .. LANDED_AT + 30 (B's reads sit behind odd ones); done well
       // before the period ends, where the next one's first barrier waits for them
       if constexpr (m >= LANDED_AT && m < LANDED_AT + 32 && (m % 2) == 0) {
         constexpr int j = (m - LANDED_AT) / 2, ii = j / 2, kk = j % 2;
         fa[par ^ 1][ii][kk] = fra.read((par ^ 1) * 32768, ii, kk);
       }
-      // ---- loads behind it: all sixteen in the first half, A's tile q+2 over tile q, B's over tile q-1
+      // ---- loads behind it: one every LOAD_STEP MFMAs, A's tile q+2 over tile q, then B's over tile q-1
       if constexpr (m >= 2 && (m - 2) % LOAD_STEP == 0 && (m - 2) / LOAD_STEP < IA + LB) {
         constexpr int l = (m - 2) / LOAD_STEP;
         if constexpr (l < IA) load_a(std::integral_constant<int, l>{}, par * 32768);

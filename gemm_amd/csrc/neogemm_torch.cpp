@@ -45,9 +45,26 @@ struct WorkspaceKey {
   hipStream_t stream;
   bool operator<(const WorkspaceKey& o) const { return device != o.device ? device < o.device : stream < o.stream; }
 };
+// At most kMaxWorkspaces buffers are kept: streams come and go, and a buffer whose stream is gone would otherwise stay
+// for the life of the thread.  The least recently used one is dropped (safe for the reason above).
+constexpr size_t kMaxWorkspaces = 16;
+struct WorkspaceSlot {
+  torch::Tensor buffer;
+  uint64_t last_use = 0;
+};
 torch::Tensor& workspace_for(const torch::Tensor& like, hipStream_t stream, size_t bytes) {
-  static thread_local std::map<WorkspaceKey, torch::Tensor> ws;
-  torch::Tensor& t = ws[WorkspaceKey{(int)like.get_device(), stream}];
+  static thread_local std::map<WorkspaceKey, WorkspaceSlot> ws;
+  static thread_local uint64_t clock = 0;
+  const WorkspaceKey key{(int)like.get_device(), stream};
+  if (ws.find(key) == ws.end() && ws.size() >= kMaxWorkspaces) {
+    auto oldest = ws.begin();
+    for (auto it = ws.begin(); it != ws.end(); ++it)
+      if (it->second.last_use < oldest->second.last_use) oldest = it;
+    ws.erase(oldest);
+  }
+  WorkspaceSlot& slot = ws[key];
+  slot.last_use = ++clock;
+  torch::Tensor& t = slot.buffer;
   if (!t.defined() || (size_t)t.numel() < bytes) {
     t = torch::Tensor();  // give the old block back first
     t = torch::empty({(int64_t)bytes}, like.options().dtype(torch::kUInt8));

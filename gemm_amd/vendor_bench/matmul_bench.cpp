@@ -9,8 +9,11 @@
 //
 //   matmul_bench M N K [reps=100] [b_layout=0|1] [variant=0] [split_k=0] [group_m=0] [nbuf=1]
 //   matmul_bench ceiling [preheat_ms=1000]
+//   matmul_bench loadpath M N K [b_layout=1] [strip=64]
 //
-// One line of JSON per library on stdout.
+// One line of JSON per library on stdout.  Lines of timed runs carry "t0" / "t1", CLOCK_MONOTONIC seconds around the
+// timed batches, so that a parent process that samples the board's power and clocks can tell which samples belong to
+// which run.
 //
 // `ceiling` measures what the matrix cores sustain with nothing else going on: every wave runs the MFMA
 // sequence of a 128x128 wave tile (the 256x256 GEMM tile's share of one wave) from registers, no memory
@@ -20,9 +23,16 @@
 // the data-sheet peak, bounds any GEMM kernel on such inputs on this chip.
 // It then runs the 128 MFMAs of a wave tile in four different orders (mfma_order_kernel) and the sequence next to the
 // other activities of a GEMM main loop (gemm_like_kernel): what each costs at the power limit.
+//
+// `loadpath` measures the path into the CUs of a decode-shaped GEMM (few rows M, all of B read once) with the arithmetic
+// taken away: every workgroup requests its strip of B (from HBM; B rotates through buffers larger than the last-level
+// cache) and all of A (from L2), by global->LDS loads of whole 128-byte lines, and nothing else: no LDS reads, no MFMAs,
+// no C.  What that takes bounds every kernel that gives a workgroup a strip of columns and all of K.
 #include <hip/hip_runtime.h>
 #include <hipblaslt/hipblaslt.h>
 #include <rocblas/rocblas.h>
+
+#include <time.h>
 
 #include <algorithm>
 #include <cmath>
@@ -73,6 +83,13 @@ static double preheat_ms_from_env() {
   return e ? atof(e) : 0.0;
 }
 
+static double monotonic_s() {
+  timespec ts;
+  clock_gettime(CLOCK_MONOTONIC, &ts);
+  return (double)ts.tv_sec + 1e-9 * (double)ts.tv_nsec;
+}
+static double g_t0 = 0.0, g_t1 = 0.0;  // CLOCK_MONOTONIC around the timed batches of the last time_ms()
+
 template <class F>
 static double time_ms(F&& launch, int reps, hipStream_t st) {
   hipEvent_t a, b;
@@ -93,6 +110,7 @@ static double time_ms(F&& launch, int reps, hipStream_t st) {
   }
   // median of 5 batches
   std::vector<double> ms;
+  g_t0 = monotonic_s();
   for (int batch = 0; batch < 5; ++batch) {
     HIP_OK(hipEventRecord(a, st));
     for (int i = 0; i < reps; ++i) launch(i);
@@ -102,6 +120,7 @@ static double time_ms(F&& launch, int reps, hipStream_t st) {
     HIP_OK(hipEventElapsedTime(&t, a, b));
     ms.push_back(t / reps);
   }
+  g_t1 = monotonic_s();
   std::sort(ms.begin(), ms.end());
   HIP_OK(hipEventDestroy(a));
   HIP_OK(hipEventDestroy(b));
@@ -111,9 +130,9 @@ static double time_ms(F&& launch, int reps, hipStream_t st) {
 static void report(const char* lib, int64_t M, int64_t N, int64_t K, int bl, double ms, const char* extra) {
   const double flop = 2.0 * M * N * K, bytes = 2.0 * (M * K + K * N + M * N);
   printf("{\"lib\": \"%s\", \"M\": %lld, \"N\": %lld, \"K\": %lld, \"b_layout\": %d, \"ms\": %.5f, \"tflops\": %.2f, "
-         "\"pct_of_2500\": %.2f, \"gbps\": %.1f, \"pct_of_8000\": %.2f%s}\n",
+         "\"pct_of_2500\": %.2f, \"gbps\": %.1f, \"pct_of_8000\": %.2f, \"t0\": %.4f, \"t1\": %.4f%s}\n",
          lib, (long long)M, (long long)N, (long long)K, bl, ms, flop / ms / 1e9, flop / ms / 1e9 / 25.0,
-         bytes / ms / 1e6, bytes / ms / 1e6 / 80.0, extra);
+         bytes / ms / 1e6, bytes / ms / 1e6 / 80.0, g_t0, g_t1, extra);
   fflush(stdout);
 }
 
@@ -385,8 +404,8 @@ static int run_ceiling(int preheat_ms) {
     // with 64 (16) independent accumulators a wave issues MFMAs back to back: 16 (32) cycles each, 1024 flop per
     // cycle and SIMD, so the rate implies the clock the chip held
     printf("{\"ceiling\": \"%s\", \"operands\": \"%s\", \"ms\": %.5f, \"tflops\": %.1f, \"pct_of_2500\": %.2f, "
-           "\"implied_mhz\": %.0f, \"workgroups\": %d, \"waves_per_simd\": 1}\n",
-           c.insn, c.data, ms, tflops, tflops / 25.0, tflops * 1e12 / (256.0 * 4 * 1024.0) / 1e6, wgs);
+           "\"implied_mhz\": %.0f, \"workgroups\": %d, \"waves_per_simd\": 1, \"t0\": %.4f, \"t1\": %.4f}\n",
+           c.insn, c.data, ms, tflops, tflops / 25.0, tflops * 1e12 / (256.0 * 4 * 1024.0) / 1e6, wgs, g_t0, g_t1);
     fflush(stdout);
   }
   // the order of the MFMAs of a wave tile, N(0,1) operands
@@ -415,7 +434,8 @@ static int run_ceiling(int preheat_ms) {
       const double ms = time_ms(launch, 40, st);
       const double tflops = flop / ms / 1e9;
       printf("{\"ceiling\": \"mfma_order\", \"order\": \"%s\", \"operands\": \"%s\", \"ms\": %.5f, \"tflops\": %.1f, "
-             "\"pct_of_2500\": %.2f}\n", o.name, zero ? "zeros" : "randn", ms, tflops, tflops / 25.0);
+             "\"pct_of_2500\": %.2f, \"t0\": %.4f, \"t1\": %.4f}\n", o.name, zero ? "zeros" : "randn", ms, tflops, tflops / 25.0,
+             g_t0, g_t1);
       fflush(stdout);
     }
   }
@@ -458,18 +478,97 @@ static int run_ceiling(int preheat_ms) {
       const double ms = time_ms(launch, 40, st);
       const double tflops = flop / ms / 1e9;
       printf("{\"ceiling\": \"gemm_like\", \"parts\": \"%s\", \"operands\": \"%s\", \"ms\": %.5f, \"tflops\": %.1f, "
-             "\"pct_of_2500\": %.2f}\n", l.name, zero ? "zeros" : "randn", ms, tflops, tflops / 25.0);
+             "\"pct_of_2500\": %.2f, \"t0\": %.4f, \"t1\": %.4f}\n", l.name, zero ? "zeros" : "randn", ms, tflops, tflops / 25.0,
+             g_t0, g_t1);
       fflush(stdout);
     }
   }
   return 0;
 }
 
+// ---- load path of a decode-shaped GEMM, arithmetic taken away ---------------------------------------
+// One 128-deep step of a workgroup: B 2 * strip / 8 requests (8 rows x 128 B each; B [K,N]: 16 requests of 8 k-rows x
+// 128 B), A 2 * M / 8 requests.  The NW waves take the requests of a step round-robin; each keeps at most D in flight.
+typedef __attribute__((ext_vector_type(4))) int ci32x4b;
+template <int D>
+__global__ __launch_bounds__(512) void loadpath_kernel(const char* A, const char* B, float* out, int M, int K, int N, int strip,
+                                                       int with_a, int b_kn) {
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  const uint32_t l0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), nw = blockDim.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const uint64_t bb = b_kn ? (uint64_t)B + (uint64_t)blockIdx.x * strip * 2 : (uint64_t)B + (uint64_t)blockIdx.x * strip * K * 2;
+  const uint32_t ldb = b_kn ? (uint32_t)N * 2 : (uint32_t)K * 2;
+  const uint32_t voff_b = (lane >> 3) * ldb + (lane & 7) * 16, voff_a = (lane >> 3) * (uint32_t)K * 2 + (lane & 7) * 16;
+  asm volatile("s_mov_b32 m0, %0" ::"s"(l0 + wave * 1024) : "memory");
+  const int nb = b_kn ? 16 : strip / 8 * 2, na = with_a ? (M + 7) / 8 * 2 : 0;
+  for (int s = 0; s < K / 128; ++s) {
+    for (int r = wave; r < nb + na; r += nw) {
+      const bool isb = r < nb;
+      const int q = isb ? r : r - nb;
+      // the request's first byte; lanes past the matrix (rows of A beyond M) read as zeros
+      uint64_t base;
+      uint32_t limit;
+      if (isb && b_kn) base = bb + ((uint64_t)s * 128 + (uint64_t)q * 8) * ldb, limit = 7 * ldb + 128;
+      else if (isb) base = bb + (uint64_t)(q >> 1) * 8 * ldb + (q & 1) * 128 + (uint64_t)s * 256, limit = 7 * ldb + 128;
+      else {
+        base = (uint64_t)A + (uint64_t)(q >> 1) * 8 * K * 2 + (q & 1) * 128 + (uint64_t)s * 256;
+        const int rows = M - (q >> 1) * 8 < 8 ? M - (q >> 1) * 8 : 8;
+        limit = (uint32_t)(rows - 1) * K * 2 + 128;
+      }
+      const ci32x4b rs = {(int)(uint32_t)base, (int)((base >> 32) & 0xffff), (int)limit, 0x00020000};
+      asm volatile("buffer_load_dwordx4 %0, %1, 0 offen sc1 lds" ::"v"(isb ? voff_b : voff_a), "s"(rs) : "memory");
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(D) : "memory");
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  out[blockIdx.x * blockDim.x + threadIdx.x] = ((float*)smem)[threadIdx.x];
+}
+
+static int run_loadpath(int64_t M, int64_t N, int64_t K, int b_layout, int strip) {
+  if (M < 1 || N < strip || K < 128 || K % 128 || N % strip || strip % 8 || strip > 64 || (b_layout == 0 && strip != 64)) {
+    fprintf(stderr, "loadpath: K a multiple of 128, N a multiple of the strip (a multiple of 8 up to 64; 64 with B [K,N])\n");
+    return 2;
+  }
+  hipStream_t st;
+  HIP_OK(hipStreamCreate(&st));
+  const size_t b_bytes = (size_t)N * K * 2;
+  const int nbuf = (int)std::min<size_t>(8, (1ull << 30) / b_bytes + 1);
+  void *dA, *dout;
+  std::vector<void*> dB(nbuf);
+  HIP_OK(hipMalloc(&dA, (size_t)M * K * 2));
+  HIP_OK(hipMemset(dA, 1, (size_t)M * K * 2));
+  for (auto& p : dB) {
+    HIP_OK(hipMalloc(&p, b_bytes));
+    HIP_OK(hipMemset(p, 1, b_bytes));
+  }
+  const int wgs = (int)(N / strip);
+  HIP_OK(hipMalloc(&dout, (size_t)wgs * 512 * 4));
+  HIP_OK(hipFuncSetAttribute((const void*)loadpath_kernel<16>, hipFuncAttributeMaxDynamicSharedMemorySize, 65536));
+  for (int with_a = 0; with_a < 2; ++with_a)
+    for (int threads : {256, 512}) {
+      auto launch = [&](int i) {
+        loadpath_kernel<16><<<wgs, threads, 65536, st>>>((const char*)dA, (const char*)dB[i % nbuf], (float*)dout, (int)M, (int)K, (int)N, strip,
+                                                         with_a, b_layout == 0);
+      };
+      const double ms = time_ms(launch, 100, st);
+      HIP_OK(hipGetLastError());
+      printf("{\"loadpath\": \"%s\", \"M\": %lld, \"N\": %lld, \"K\": %lld, \"b_layout\": %d, \"strip\": %d, \"workgroups\": %d, "
+             "\"waves\": %d, \"requests_in_flight_per_wave\": 16, \"us\": %.2f, \"b_tbps\": %.2f, \"a_from_l2_mb\": %.1f}\n",
+             with_a ? "B from HBM + all of A from L2 per workgroup" : "B from HBM only", (long long)M, (long long)N, (long long)K,
+             b_layout, strip, wgs, threads / 64, ms * 1e3, (double)b_bytes / ms / 1e9, with_a ? (double)wgs * M * K * 2 / 1e6 : 0.0);
+      fflush(stdout);
+    }
+  return 0;
+}
+
 int main(int argc, char** argv) {
   if (argc >= 2 && strcmp(argv[1], "ceiling") == 0) return run_ceiling(argc > 2 ? atoi(argv[2]) : 1000);
+  if (argc >= 5 && strcmp(argv[1], "loadpath") == 0)
+    return run_loadpath(atoll(argv[2]), atoll(argv[3]), atoll(argv[4]), argc > 5 ? atoi(argv[5]) : 1, argc > 6 ? atoi(argv[6]) : 64);
   if (argc < 4) {
-    fprintf(stderr, "usage: %s M N K [reps] [b_layout] [variant] [split_k] [group_m] [nbuf]\n       %s ceiling [preheat_ms]\n",
-            argv[0], argv[0]);
+    fprintf(stderr, "usage: %s M N K [reps] [b_layout] [variant] [split_k] [group_m] [nbuf]\n       %s ceiling [preheat_ms]\n"
+            "       %s loadpath M N K [b_layout] [strip]\n", argv[0], argv[0], argv[0]);
     return 2;
   }
   const int64_t M = atoll(argv[1]), N = atoll(argv[2]), K = atoll(argv[3]);

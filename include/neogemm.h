@@ -130,7 +130,10 @@ size_t neogemm_bf16_batched_workspace_bytes(int64_t M, int64_t N, int64_t K, int
  * loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same arguments and
  * result as neogemm_bf16 (bit for bit: the same kernels run), minus the workspace: split-K partials go to
  * an array of NEOGEMM_NOALLOC_SCRATCH_BYTES that the library's code object holds on each GPU it runs on,
- * until the process ends.  The call makes no hipMalloc/hipFree and no other allocating call.  A shape whose
+ * until the process ends.  The call makes no hipMalloc/hipFree and no other allocating call; the first call on a
+ * device (it resolves the array's address, which loads the code object) and the first launch of a kernel instance (it
+ * raises that kernel's dynamic-LDS limit) make host-side set-up calls that a capturing stream does not allow: warm the
+ * shapes up once outside the capture, then capture.  A shape whose
  * neogemm_bf16_workspace_bytes(M,N,K) exceeds NEOGEMM_NOALLOC_SCRATCH_BYTES is refused with
  * NEOGEMM_ERR_SCRATCH_LIMIT and nothing is launched.  All calls on one GPU share that GPU's array: calls on
  * one stream are ordered and safe (every partial is rewritten before it is read, nothing has to start at

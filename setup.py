@@ -67,6 +67,7 @@ if __name__ == "__main__":
             CppExtension(
                 name="neoGEMM",
                 sources=["gemm_amd/csrc/neogemm_torch.cpp"],
+                depends=[os.path.join("include", "neogemm.h")],   # the shim is rebuilt when the C ABI changes
                 include_dirs=[os.path.join(ROOT, "include"), os.path.join(ROCM, "include")],
                 define_macros=[("__HIP_PLATFORM_AMD__", "1"), ("USE_ROCM", "1")],
                 extra_compile_args=["-std=c++17", "-O2", "-Wno-unused-result"],

@@ -115,11 +115,15 @@ def test_workspace_query_bounds_every_layout():
     for M, N, K in ((1024, 6144, 8192), (2048, 3072, 8192), (512, 6144, 8192), (4096, 1536, 8192)):
         v, s = _abi.plan(M, N, K, _abi.B_NK, _abi.C_COL)
         assert _abi.workspace_bytes(M, N, K) >= (s * M * N * 4 if s > 1 else 0)
-    # batched query likewise
+    # the batched query: a batch of one is the plain query; a larger batch asks for whole sets of fp32 partials (that the
+    # queried size carries every layout pair's batched call is checked on the GPU, tests/test_gemm_gpu.py)
     lib = _abi.load()
-    for batch in (2, 7):
-        for M, N, K in ((128, 128, 8192), (256, 512, 16384), (1024, 6144, 8192)):
-            assert lib.neogemm_bf16_batched_workspace_bytes(M, N, K, batch) >= 0
+    for M, N, K in ((128, 128, 8192), (256, 512, 16384), (1024, 6144, 8192)):
+        assert lib.neogemm_bf16_batched_workspace_bytes(M, N, K, 1) == _abi.workspace_bytes(M, N, K)
+        for batch in (2, 7):
+            need = lib.neogemm_bf16_batched_workspace_bytes(M, N, K, batch)
+            assert need % (M * N * 4 * batch) == 0 and need // (M * N * 4 * batch) in (0, 2, 3, 4, 6, 8, 12, 16, 24, 32, 48, 64)
+    assert lib.neogemm_bf16_batched_workspace_bytes(128, 128, 8192, 2) > 0
 
 
 def test_argument_validation_returns_before_touching_the_gpu():

@@ -170,29 +170,52 @@ def test_parity_512(dev, variant, b_layout, c_layout):
     o.assert_parity(got, A, Bkn, what=f"512^3 v{variant} b{b_layout} c{c_layout}")
 
 
-def check_big(dev, M, N, K, seed, b_layout=g.B_KN, variant=None, split_k=0, nrows=256):
-    """Full-size run; ulp and Frobenius against the full fp32 CPU product, the fp64-based bound on a
-    sample of rows (all rows when the problem is small)."""
+def check_big(dev, M, N, K, seed, b_layout=g.B_KN, variant=None, split_k=0, nrows=256, c_layout=g.C_ROW):
+    """Full-size run.  Over the whole matrix, against the full fp32 CPU product: raw ulp, Frobenius error and the ulp
+    measured at max(|ref|, 2^-7 rms) (see oracle.parity_report); the fp64-based bound, which needs a second full
+    product in fp64, on a sample of rows (all rows when the problem is small)."""
     A, Bkn = o.make_inputs(M, N, K, seed=seed)
-    got = run_abi(A, layouts(Bkn, b_layout), dev, b_layout, g.C_ROW, variant, split_k)
+    got = run_abi(A, layouts(Bkn, b_layout), dev, b_layout, c_layout, variant, split_k)
     ref = o.ref_gemm(A, Bkn)
     ulp = o.ulp_distance(o.bits_of(got), o.bits_of(ref))
     assert bool(torch.isfinite(got.float()).all())
     assert (ulp > 1).mean() <= 2e-3, f"{(ulp > 1).mean():.2e} of elements more than 1 raw ulp off"
-    rel = float(torch.linalg.norm(got.float() - ref.float()) / torch.linalg.norm(ref.float()))
+    rf = ref.float()
+    rel = float(torch.linalg.norm(got.float() - rf) / torch.linalg.norm(rf))
     assert rel <= o.TOL_REL_FRO, rel
+    floor = max(float(torch.sqrt(torch.mean(rf.double() ** 2))) * 2.0 ** -7, 1e-38)
+    ulp_size = torch.exp2(torch.floor(torch.log2(torch.clamp(rf.abs(), min=floor))) - 7)
+    floored = float(((got.float() - rf).abs() / ulp_size).max())
+    assert floored <= o.TOL_ULP, f"{floored} ulp (floored) over the whole {M}x{N} matrix"
     idx = torch.arange(M) if M <= nrows else torch.cat([
         torch.tensor([0, M - 1]), torch.randperm(M, generator=torch.Generator().manual_seed(seed))[:nrows - 2]])
     return o.assert_parity(got[idx], A[idx], Bkn, ref=ref[idx], what=f"{M}x{N}x{K}")
 
 
-@pytest.mark.parametrize("b_layout", [g.B_KN, g.B_NK])
-def test_parity_4096(dev, b_layout):
-    check_big(dev, 4096, 4096, 4096, seed=1, b_layout=b_layout)
+@pytest.mark.parametrize("b_layout,c_layout", [(g.B_KN, g.C_ROW), (g.B_NK, g.C_ROW), (g.B_NK, g.C_COL)])
+def test_parity_4096(dev, b_layout, c_layout):
+    check_big(dev, 4096, 4096, 4096, seed=1, b_layout=b_layout, c_layout=c_layout)
 
 
 def test_parity_8192_headline(dev):
     check_big(dev, 8192, 8192, 8192, seed=2)
+
+
+def test_parity_8192_reference_call(dev):
+    """The reference's own call at the headline size: B [N,K], column-major C (benchmark.py:10-25, nemgemmV03.cu:343-391):
+    the chained kernel on exchanged operands, four rounds of workgroups; through the C ABI and through neoGEMM.neoGemmV1."""
+    M = N = K = 8192
+    assert g.plan(M, N, K, g.B_NK, g.C_COL) == (g.VARIANT_C256x256_W4, 1)
+    check_big(dev, M, N, K, seed=3, b_layout=g.B_NK, c_layout=g.C_COL)
+    import neoGEMM
+    A, Bkn = o.make_inputs(M, N, K, seed=3)
+    Ad, Bd = A.to(dev), Bkn.t().contiguous().to(dev)
+    Cbuf = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=dev)
+    neoGEMM.neoGemmV1(Ad, Bd, Cbuf)                       # C storage receives the column-major product
+    torch.cuda.synchronize()
+    via_module = Cbuf.t().cpu()                            # benchmark.py:25
+    via_abi = run_abi(A, Bkn.t().contiguous(), dev, g.B_NK, g.C_COL)
+    assert torch.equal(via_module, via_abi)                # the same kernel on the same data, bit for bit
 
 
 @pytest.mark.parametrize("M", [16, 64, 72, 100, 128])
@@ -729,6 +752,41 @@ def test_batched_parity(dev, batch, M, N, K):
     # one problem of the batch is the plain call bit for bit when both take the same (variant, split)
     if g.plan(M, N, K) == tuple(_abi.plan(M, N, K)) and batch == 1:
         assert np.array_equal(o.bits_of(C[0].cpu()), o.bits_of(g.gemm(A[0].to(dev), B[0].to(dev)).cpu()))
+
+
+@pytest.mark.parametrize("batch", [2, 7])
+def test_batched_workspace_query_bounds_every_layout(dev, batch):
+    """A workspace of exactly neogemm_bf16_batched_workspace_bytes(M,N,K,batch) must carry the batched call in every
+    layout pair (the batched plan splits K differently from the single call's, and differently per layout): shapes
+    with few output tiles and a deep K, where the plan splits."""
+    lib = _abi.load()
+    split_somewhere = False
+    for (M, N, K) in ((128, 128, 8192), (256, 512, 16384), (64, 256, 4096), (1024, 1024, 8192)):
+        need = int(lib.neogemm_bf16_batched_workspace_bytes(M, N, K, batch))
+        split_somewhere |= need > 0
+        assert need % (M * N * 4 * batch) == 0                      # a whole number of fp32 partials per problem
+        ws = torch.empty(max(need, 16), dtype=torch.uint8, device=dev)
+        A, Bkn = o.make_inputs(batch * M, N, K, seed=batch + M)    # a batch of different A, one shared B
+        ref = o.ref_gemm(A, Bkn)
+        for b_layout in (g.B_KN, g.B_NK):
+            for c_layout in (g.C_ROW, g.C_COL):
+                Ad, Bd = A.to(dev), layouts(Bkn, b_layout).to(dev)
+                C = torch.full((batch, M, N) if c_layout == g.C_ROW else (batch, N, M), float("nan"), dtype=torch.bfloat16, device=dev)
+                st = lib.neogemm_bf16_batched(Ad.data_ptr(), Bd.data_ptr(), C.data_ptr(), M, N, K, K, N if b_layout == g.B_KN else K,
+                                              N if c_layout == g.C_ROW else M, M * K, 0, M * N, batch, b_layout, c_layout,
+                                              ws.data_ptr() if need else None, need, None)
+                assert st == _abi.OK, (M, N, K, batch, b_layout, c_layout, need, _abi.strerror(st))
+                torch.cuda.synchronize()
+                got = C.cpu() if c_layout == g.C_ROW else C.cpu().transpose(1, 2).contiguous()
+                o.assert_parity(got.reshape(batch * M, N), A, Bkn, ref=ref, what=f"batched {batch}x{M}x{N}x{K} b{b_layout} c{c_layout}")
+                if need:
+                    # one byte less is refused, never overrun (where this layout pair's plan needs all of it, or less)
+                    st = lib.neogemm_bf16_batched(Ad.data_ptr(), Bd.data_ptr(), C.data_ptr(), M, N, K, K, N if b_layout == g.B_KN else K,
+                                                  N if c_layout == g.C_ROW else M, M * K, 0, M * N, batch, b_layout, c_layout,
+                                                  ws.data_ptr(), M * N * 4 * batch - 1, None)
+                    assert st in (_abi.OK, _abi.ERR_WORKSPACE)
+                    torch.cuda.synchronize()
+    assert split_somewhere
 
 
 def test_batched_argument_checks(dev):

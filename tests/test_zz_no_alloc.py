@@ -74,3 +74,36 @@ def test_noalloc_refuses_what_does_not_fit(dev):
     assert bool((C == 7.0).all())   # nothing ran
     # the argument checks of neogemm_bf16 apply unchanged
     assert call_noalloc(A, B, C, 256, 256, 512, 5, g.C_COL) == _abi.ERR_BAD_ARG
+
+
+def test_noalloc_under_graph_capture(dev):
+    """The caller this entry point is for: a stream under HIP graph capture.  One warm-up call outside the capture (the
+    first call on a device resolves the array's address, the first launch of a kernel instance raises its LDS limit:
+    both are host-side set-up calls that a capturing stream does not allow), then the call is captured (kernel launches
+    only: the split-K tile kernel and the reduce), and every replay, with eager work and synchronisations in between
+    and fresh inputs each time, equals the eager result bit for bit."""
+    M, N, K = 264, 392, 8200
+    b_layout, c_layout = g.B_KN, g.C_ROW
+    assert g.plan(M, N, K, b_layout, c_layout)[1] > 1
+    gen = torch.Generator().manual_seed(5)
+    A0, Bkn = o.make_inputs(M, N, K, seed=50)
+    Ad, Bd = A0.to(dev), Bkn.to(dev)
+    got = torch.zeros(M, N, dtype=torch.bfloat16, device=dev)
+    eager = torch.zeros(M, N, dtype=torch.bfloat16, device=dev)
+    assert call_noalloc(Ad, Bd, eager, M, N, K, b_layout, c_layout) == _abi.OK      # warm-up, outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        st = call_noalloc(Ad, Bd, got, M, N, K, b_layout, c_layout)                 # on the capturing stream
+    assert st == _abi.OK, _abi.strerror(st)
+    for it in range(4):
+        # fresh inputs in the same buffers (eager work between the replays), then replay and eager call
+        Ad.copy_((torch.randn(M, K, generator=gen) / K ** 0.5).to(torch.bfloat16))
+        got.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert call_noalloc(Ad, Bd, eager, M, N, K, b_layout, c_layout) == _abi.OK
+        torch.cuda.synchronize()
+        assert torch.equal(got.view(torch.int16), eager.view(torch.int16)), f"replay {it}"
+    o.assert_parity(got[:64].cpu(), Ad[:64].cpu(), Bkn, what="noalloc under capture")
