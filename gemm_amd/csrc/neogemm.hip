@@ -1806,7 +1806,10 @@ static void plan_model(int64_t M, int64_t N, int64_t K, bool aligned, int c_layo
       // both operands K-major: the tall tile runs a little ahead of the wide one (2560^3: 33.8 against 35.0 us)
       if (c.variant == NEOGEMM_VARIANT_T128x256_W4 && b_layout == NEOGEMM_B_NK) t *= 1.02;
       // latency knows no discount, and two latency-bound workgroups on one CU were measured to take turns
-      const double lat_floor = __builtin_ceil(wgs / cus) * ktps * lat_us;
+      // (with both operands K-major the 128x128 tile has three tiles of each in flight when it streams: 256 x 14336 x 4096
+      // unsplit runs its 64 K tiles in 32.3 us)
+      const double lat_v = c.variant == NEOGEMM_VARIANT_T128x128_W4 && bytes > 32e6 && b_layout == NEOGEMM_B_NK ? 0.46 : lat_us;
+      const double lat_floor = __builtin_ceil(wgs / cus) * ktps * lat_v;
       if (t < lat_floor) t = lat_floor;
       t += rounds * (c.fixed_us + (sp > 1 ? c.split_fixed_us : 0.0));
       // fewer workgroups than CUs pull less from HBM: 112 of them 4.0 TB/s, 224 and more 5 and above (64x11008x14336
@@ -1969,15 +1972,33 @@ static void plan(int64_t M, int64_t N, int64_t K, bool aligned, int c_layout, in
   m.ncus = ncus;
   m.variant = *variant, m.split_k = *split_k;
 }
+// Tuned choices that ship with the library: shapes of a sweep (gemm_amd/tune.py over M in 256 .. 8192 x the (N, K) pairs of
+// common transformer layers, three layout pairs, one MI355X) where the best measured (variant, split) beat the model's
+// choice by more than 3 %.  A table named by NEOGEMM_PLAN_TABLE is looked up first; these apply on a device with the
+// CU count they were measured on.
+static const int kDefaultPlanCus = 256;
+static const PlanEntry kDefaultPlan[] = {
+#include "neogemm_default_plan.inc"
+};
 static void plan_uncached(int64_t M, int64_t N, int64_t K, bool aligned, int c_layout, int* variant, int* split_k,
                           int64_t batch, int b_layout, int ncus) {
   if (aligned && K > 0 && batch == 1) {
+    auto match = [&](const PlanEntry& e) {
+      return e.M == M && e.N == N && e.K == K && e.c_layout == c_layout && e.b_layout == b_layout;
+    };
     for (const PlanEntry& e : plan_table())
-      if (e.M == M && e.N == N && e.K == K && e.c_layout == c_layout && e.b_layout == b_layout) {
+      if (match(e)) {
         *variant = e.variant;
         *split_k = e.variant == NEOGEMM_VARIANT_GENERIC ? 1 : e.split_k;
         return;
       }
+    if (ncus == kDefaultPlanCus)
+      for (const PlanEntry& e : kDefaultPlan)
+        if (match(e)) {
+          *variant = e.variant;
+          *split_k = e.split_k;
+          return;
+        }
   }
   plan_model(M, N, K, aligned, c_layout, variant, split_k, batch, b_layout, ncus);
 }

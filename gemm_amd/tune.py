@@ -2,6 +2,7 @@
 
     python -m gemm_amd.tune --out plan_table.json 512x512x512 256x256x8192 16x14336x4096
     NEOGEMM_PLAN_TABLE=plan_table.json python bench.py        # the library reads the table once, at first use
+    python -m gemm_amd.tune --merge a.json b.json --inc gemm_amd/csrc/neogemm_default_plan.inc   # the table the library ships
 
 The table is the JSON array libneogemm.so looks up before its cost model (neogemm_bf16_plan): objects
 {"M","N","K","b_layout","c_layout","variant","split_k"}; an entry applies to exactly its shape and layouts
@@ -23,7 +24,7 @@ from ._abi import B_KN, B_NK, C_COL, C_ROW, ERR_UNSUPPORTED, NeoGemmError
 CANDIDATE_VARIANTS = (_abi.VARIANT_T256x256_W4, _abi.VARIANT_C256x256_W4, _abi.VARIANT_T256x256_W8, _abi.VARIANT_T128x256_W4,
                       _abi.VARIANT_T256x128_W4, _abi.VARIANT_T128x128_W4, _abi.VARIANT_T64x128_W4,
                       _abi.VARIANT_T192x256_W4, _abi.VARIANT_T96x128_W4, _abi.VARIANT_T64x64_W4, _abi.VARIANT_SKINNY16, _abi.VARIANT_SKINNY32, _abi.VARIANT_SKINNY64,
-                      _abi.VARIANT_SKINNY128)
+                      _abi.VARIANT_SKINNY128, _abi.VARIANT_STRIP)
 CANDIDATE_SPLITS = (1, 2, 3, 4, 6, 8, 12, 16, 24, 32)
 
 
@@ -73,6 +74,9 @@ def tune_shape(M, N, K, nbuf=1, log=sys.stderr, b_layout=B_KN, c_layout=C_ROW):
             if s > 1 and K // (64 * s) < 2:
                 break
             try:
+                # a short look first: a candidate a quarter behind the best so far is not worth a preheated measurement
+                if time_us(lambda: call(v, s), warmup=2, iters=6) > 1.25 * t_best:
+                    continue
                 t = time_us(lambda: call(v, s), preheat_ms=heat)
             except NeoGemmError as e:
                 if e.status != ERR_UNSUPPORTED:
@@ -87,15 +91,48 @@ def tune_shape(M, N, K, nbuf=1, log=sys.stderr, b_layout=B_KN, c_layout=C_ROW):
     return model, t_model, best, t_best
 
 
+def write_inc(tables, path):
+    """Merge plan tables (lists of entries as this module writes them) into the initialiser list the library compiles in
+    as its default table (gemm_amd/csrc/neogemm_default_plan.inc)."""
+    seen, rows = set(), []
+    for t in tables:
+        for e in t:
+            key = (e["M"], e["N"], e["K"], e.get("b_layout", 0), e.get("c_layout", 0))
+            if key not in seen:
+                seen.add(key)
+                rows.append(key + (e["variant"], e["split_k"]))
+    rows.sort(key=lambda r: (r[3], r[4], r[0], r[1], r[2]))
+    with open(path, "w") as f:
+        f.write("// {M, N, K, b_layout, c_layout, variant, split_k}: tuned exceptions to plan_model (see kDefaultPlan in neogemm.hip).\n"
+                "// Written by `python -m gemm_amd.tune --merge ... --inc` from the tables a tuning sweep produced; the entry with all\n"
+                "// fields zero keeps the array non-empty.\n{0, 0, 0, 0, 0, 0, 0},\n")
+        for r in rows:
+            f.write("{%d, %d, %d, %d, %d, %d, %d},\n" % r)
+    return len(rows)
+
+
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
-    ap.add_argument("shapes", nargs="+", help="MxNxK")
-    ap.add_argument("--out", required=True)
+    ap.add_argument("shapes", nargs="*", help="MxNxK")
+    ap.add_argument("--out")
+    ap.add_argument("--merge", nargs="+", metavar="TABLE.json", help="merge these tables instead of measuring (no GPU needed)")
+    ap.add_argument("--inc", help="with --merge: write the merged table as the library's default-plan include file")
     ap.add_argument("--margin", type=float, default=0.03, help="minimum relative gain over the model's choice")
     ap.add_argument("--nbuf", type=int, default=1, help="rotate this many B buffers (streaming shapes)")
     ap.add_argument("--b-layout", type=int, default=B_KN, choices=(B_KN, B_NK), help="0: B [K,N], 1: B [N,K]")
     ap.add_argument("--c-layout", type=int, default=C_ROW, choices=(C_ROW, C_COL), help="0: row-major C, 1: column-major")
     args = ap.parse_args()
+    if args.merge:
+        if not args.inc:
+            sys.exit("--merge needs --inc")
+        tables = []
+        for path in args.merge:
+            with open(path) as f:
+                tables.append(json.load(f))
+        print(f"{write_inc(tables, args.inc)} entries written to {args.inc}", file=sys.stderr)
+        return
+    if not args.shapes or not args.out:
+        sys.exit("give shapes and --out (or --merge ... --inc ...)")
     if not torch.cuda.is_available():
         sys.exit("tuning needs a GPU")
     table = []
@@ -105,8 +142,9 @@ def main():
         if best != model and t_best < t_model * (1.0 - args.margin):
             table.append({"M": M, "N": N, "K": K, "b_layout": args.b_layout, "c_layout": args.c_layout,
                           "variant": best[0], "split_k": best[1]})
-    with open(args.out, "w") as f:
-        json.dump(table, f, indent=1)
+        # the table so far after every shape: a sweep that is cut short keeps what it has measured
+        with open(args.out, "w") as f:
+            json.dump(table, f, indent=1)
     print(f"{len(table)} entries written to {args.out}", file=sys.stderr)
 
 

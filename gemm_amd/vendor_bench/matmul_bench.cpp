@@ -497,27 +497,27 @@ __global__ __launch_bounds__(512) void loadpath_kernel(const char* A, const char
   const uint32_t l0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), nw = blockDim.x >> 6;
   const int lane = threadIdx.x & 63;
+  // one buffer resource per operand; a request is told apart by a scalar offset.  Lanes past the end of A (rows beyond
+  // M) are out of the resource's range: they read as zeros and touch no memory.
   const uint64_t bb = b_kn ? (uint64_t)B + (uint64_t)blockIdx.x * strip * 2 : (uint64_t)B + (uint64_t)blockIdx.x * strip * K * 2;
   const uint32_t ldb = b_kn ? (uint32_t)N * 2 : (uint32_t)K * 2;
+  const ci32x4b ra = {(int)(uint32_t)(uint64_t)A, (int)(((uint64_t)A >> 32) & 0xffff), (int)((uint32_t)M * K * 2), 0x00020000};
   const uint32_t voff_b = (lane >> 3) * ldb + (lane & 7) * 16, voff_a = (lane >> 3) * (uint32_t)K * 2 + (lane & 7) * 16;
   asm volatile("s_mov_b32 m0, %0" ::"s"(l0 + wave * 1024) : "memory");
   const int nb = b_kn ? 16 : strip / 8 * 2, na = with_a ? (M + 7) / 8 * 2 : 0;
   for (int s = 0; s < K / 128; ++s) {
+    // B [N,K]: the strip's rows, 256 bytes further along K per step; B [K,N]: 128 k-rows further down per step
+    const uint64_t bs = b_kn ? bb + (uint64_t)s * 128 * ldb : bb + (uint64_t)s * 256;
+    const ci32x4b rb = {(int)(uint32_t)bs, (int)((bs >> 32) & 0xffff), (int)0x7fffffff, 0x00020000};
     for (int r = wave; r < nb + na; r += nw) {
-      const bool isb = r < nb;
-      const int q = isb ? r : r - nb;
-      // the request's first byte; lanes past the matrix (rows of A beyond M) read as zeros
-      uint64_t base;
-      uint32_t limit;
-      if (isb && b_kn) base = bb + ((uint64_t)s * 128 + (uint64_t)q * 8) * ldb, limit = 7 * ldb + 128;
-      else if (isb) base = bb + (uint64_t)(q >> 1) * 8 * ldb + (q & 1) * 128 + (uint64_t)s * 256, limit = 7 * ldb + 128;
-      else {
-        base = (uint64_t)A + (uint64_t)(q >> 1) * 8 * K * 2 + (q & 1) * 128 + (uint64_t)s * 256;
-        const int rows = M - (q >> 1) * 8 < 8 ? M - (q >> 1) * 8 : 8;
-        limit = (uint32_t)(rows - 1) * K * 2 + 128;
+      if (r < nb) {
+        const uint32_t soff = b_kn ? (uint32_t)r * 8 * ldb : (uint32_t)(r >> 1) * 8 * ldb + (r & 1) * 128;
+        asm volatile("buffer_load_dwordx4 %0, %1, %2 offen sc1 lds" ::"v"(voff_b), "s"(rb), "s"(soff) : "memory");
+      } else {
+        const int q = r - nb;
+        const uint32_t soff = (uint32_t)(q >> 1) * 8 * K * 2 + (q & 1) * 128 + (uint32_t)s * 256;
+        asm volatile("buffer_load_dwordx4 %0, %1, %2 offen sc1 lds" ::"v"(voff_a), "s"(ra), "s"(soff) : "memory");
       }
-      const ci32x4b rs = {(int)(uint32_t)base, (int)((base >> 32) & 0xffff), (int)limit, 0x00020000};
-      asm volatile("buffer_load_dwordx4 %0, %1, 0 offen sc1 lds" ::"v"(isb ? voff_b : voff_a), "s"(rs) : "memory");
       asm volatile("s_waitcnt vmcnt(%0)" ::"n"(D) : "memory");
     }
   }

@@ -189,3 +189,28 @@ def test_plan_table_overrides_the_model(tmp_path):
     out = subprocess.run([sys.executable, "-c", "from gemm_amd import _abi\nprint(_abi.plan(512, 512, 512))"], env=env,
                          cwd=ROOT, capture_output=True, text=True, check=True).stdout
     assert out.strip() == str(model[0])
+
+
+def test_shipped_plan_table():
+    """The tuned exceptions compiled into the library (gemm_amd/csrc/neogemm_default_plan.inc): every entry names a kernel
+    variant the planner may return and a sensible split, the planner returns it for exactly that shape and layout pair (and
+    not for the others), and the workspace query covers its split."""
+    import re
+    inc = os.path.join(ROOT, "gemm_amd", "csrc", "neogemm_default_plan.inc")
+    rows = [tuple(int(x) for x in m.groups()) for m in
+            re.finditer(r"^\{(\d+), (\d+), (\d+), (\d+), (\d+), (\d+), (\d+)\},", open(inc).read(), re.M)]
+    rows = [r for r in rows if r[0] > 0]
+    assert len(rows) >= 10
+    assert len({r[:5] for r in rows}) == len(rows)                       # one entry per shape and layout pair
+    tile_variants = (_abi.VARIANT_T256x256_W4, _abi.VARIANT_T128x128_W4, _abi.VARIANT_T256x128_W4, _abi.VARIANT_T128x256_W4,
+                     _abi.VARIANT_T64x128_W4, _abi.VARIANT_T192x256_W4, _abi.VARIANT_T96x128_W4, _abi.VARIANT_T64x64_W4,
+                     _abi.VARIANT_C256x256_W4, _abi.VARIANT_T256x256_W8)
+    for (M, N, K, b, c, v, s) in rows:
+        assert b in (0, 1) and c in (0, 1) and 1 <= s <= 64 and s * 128 <= K
+        assert v in tile_variants + (_abi.VARIANT_SKINNY16, _abi.VARIANT_SKINNY32, _abi.VARIANT_SKINNY64, _abi.VARIANT_SKINNY128,
+                                     _abi.VARIANT_STRIP)
+        if v in (_abi.VARIANT_C256x256_W4, _abi.VARIANT_STRIP) or v >= _abi.VARIANT_SKINNY16 and v <= _abi.VARIANT_SKINNY64:
+            assert s == 1
+        assert _abi.plan(M, N, K, b, c) == (v, s), (M, N, K, b, c)
+        assert _abi.workspace_bytes(M, N, K) >= (s * M * N * 4 if s > 1 else 0)
+        assert _abi.plan(M, N, K, b, c, aligned=False) == (_abi.VARIANT_GENERIC, 1)   # the table is for the MFMA path only
