@@ -77,8 +77,8 @@ def vendor_leg(M, N, K, preheat_ms, sampler=None):
 
 def brief(summary):
     """mean socket power and shader clock of a telemetry summary, for the per-leg tables"""
-    if not summary.get("available") or not summary.get("samples"):
-        return None
+    if not summary.get("available") or summary.get("samples", 0) < 8:
+        return None   # the board refreshes its readings every few tens of milliseconds: a leg shorter than that says nothing
     return {"socket_power_w": summary.get("socket_power_w", {}).get("mean"),
             "shader_clock_mhz": summary.get("shader_clock_mhz", {}).get("mean"), "samples": summary["samples"]}
 

@@ -1807,8 +1807,9 @@ static void plan_model(int64_t M, int64_t N, int64_t K, bool aligned, int c_layo
       if (c.variant == NEOGEMM_VARIANT_T128x256_W4 && b_layout == NEOGEMM_B_NK) t *= 1.02;
       // latency knows no discount, and two latency-bound workgroups on one CU were measured to take turns
       // (with both operands K-major the 128x128 tile has three tiles of each in flight when it streams: 256 x 14336 x 4096
-      // unsplit runs its 64 K tiles in 32.3 us)
-      const double lat_v = c.variant == NEOGEMM_VARIANT_T128x128_W4 && bytes > 32e6 && b_layout == NEOGEMM_B_NK ? 0.46 : lat_us;
+      // unsplit, 224 workgroups, runs its 64 K tiles in 32.3 us; with far fewer workgroups than CUs a K tile takes longer)
+      const double lat_v =
+          c.variant == NEOGEMM_VARIANT_T128x128_W4 && bytes > 32e6 && b_layout == NEOGEMM_B_NK && wgs >= 0.6 * cus ? 0.46 : lat_us;
       const double lat_floor = __builtin_ceil(wgs / cus) * ktps * lat_v;
       if (t < lat_floor) t = lat_floor;
       t += rounds * (c.fixed_us + (sp > 1 ? c.split_fixed_us : 0.0));
