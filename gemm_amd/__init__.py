@@ -13,8 +13,8 @@ import torch
 from . import _abi
 from ._abi import (B_KN, B_NK, C_COL, C_ROW, NeoGemmError, VARIANT_AUTO, VARIANT_GENERIC, VARIANT_NAMES,  # noqa: F401
                    VARIANT_SKINNY16, VARIANT_SKINNY32, VARIANT_SKINNY64, VARIANT_SKINNY128, VARIANT_STRIP, VARIANT_T192x256_W4, VARIANT_T96x128_W4, VARIANT_T64x64_W4, VARIANT_C256x256_W4,
-                   VARIANT_T128x128_W4, VARIANT_T128x128_W4S, VARIANT_T128x256_W4, VARIANT_T256x128_W4, VARIANT_T256x256_W4,
-                   VARIANT_T256x256_W8, VARIANT_T64x128_W4, plan, strerror, version, workspace_bytes)
+                   VARIANT_T128x128_W4, VARIANT_T128x256_W4, VARIANT_T256x128_W4, VARIANT_T256x256_W4,
+                   VARIANT_T64x128_W4, plan, strerror, version, workspace_bytes)
 
 __all__ = ["gemm", "neoGemmV1", "neogemm", "gemm_into", "plan", "workspace_bytes", "version", "NeoGemmError"]
 

@@ -14,9 +14,9 @@ NOALLOC_SCRATCH_BYTES = 32 * 1024 * 1024
 B_KN, B_NK = 0, 1
 C_ROW, C_COL = 0, 1
 VARIANT_AUTO, VARIANT_GENERIC = 0, 1
-VARIANT_T256x256_W8, VARIANT_T256x256_W4, VARIANT_T128x128_W4 = 2, 3, 4
+VARIANT_T256x256_W4, VARIANT_T128x128_W4 = 3, 4   # 2 and 8 are retired numbers: the library refuses them
 VARIANT_T256x128_W4, VARIANT_T128x256_W4 = 5, 6
-VARIANT_T64x128_W4, VARIANT_T128x128_W4S = 7, 8
+VARIANT_T64x128_W4 = 7
 VARIANT_SKINNY16, VARIANT_SKINNY32, VARIANT_SKINNY64 = 9, 10, 11
 VARIANT_T192x256_W4 = 12
 VARIANT_T96x128_W4, VARIANT_T64x64_W4 = 13, 14
@@ -24,8 +24,8 @@ VARIANT_C256x256_W4 = 15
 VARIANT_SKINNY128 = 16
 VARIANT_STRIP = 17
 VARIANT_COUNT = 18
-VARIANT_NAMES = {0: "auto", 1: "generic", 2: "256x256_w8", 3: "256x256_w4", 4: "128x128_w4", 5: "256x128_w4",
-                 6: "128x256_w4", 7: "64x128_w4", 8: "128x128_w4s", 9: "skinny16", 10: "skinny32", 11: "skinny64", 12: "192x256_w4", 13: "96x128_w4", 14: "64x64_w4",
+VARIANT_NAMES = {0: "auto", 1: "generic", 2: "retired", 3: "256x256_w4", 4: "128x128_w4", 5: "256x128_w4",
+                 6: "128x256_w4", 7: "64x128_w4", 8: "retired", 9: "skinny16", 10: "skinny32", 11: "skinny64", 12: "192x256_w4", 13: "96x128_w4", 14: "64x64_w4",
                  15: "256x256_w4_chain", 16: "skinny128", 17: "strip"}
 
 # every symbol include/neogemm.h declares, with its prototype

@@ -1117,18 +1117,14 @@ NEOGEMM_TILE(256, 256, 2, 2)
 extern NEOGEMM_TILE(256, 256, 2, 2)
 #endif
 #if NEOGEMM_PART == 2
-NEOGEMM_TILE(256, 256, 2, 4)
 NEOGEMM_TILE(64, 128, 1, 4)
 #else
-extern NEOGEMM_TILE(256, 256, 2, 4)
 extern NEOGEMM_TILE(64, 128, 1, 4)
 #endif
 #if NEOGEMM_PART == 3
 NEOGEMM_TILE(128, 128, 2, 2)
-NEOGEMM_TILE(128, 128, 1, 4)
 #else
 extern NEOGEMM_TILE(128, 128, 2, 2)
-extern NEOGEMM_TILE(128, 128, 1, 4)
 #endif
 #if NEOGEMM_PART == 4
 NEOGEMM_TILE(256, 128, 2, 2)
@@ -1718,10 +1714,13 @@ struct VariantInfo {
   int bm, bn, nwaves;
 };
 static const VariantInfo kVariants[NEOGEMM_VARIANT_COUNT] = {
-    {0, 0, 0}, {16, 16, 4}, {256, 256, 8}, {256, 256, 4}, {128, 128, 4}, {256, 128, 4}, {128, 256, 4}, {64, 128, 4}, {128, 128, 4},
+    {0, 0, 0}, {16, 16, 4}, {0, 0, 0}, {256, 256, 4}, {128, 128, 4}, {256, 128, 4}, {128, 256, 4}, {64, 128, 4}, {0, 0, 0},
     {16, 64, 4}, {32, 64, 4}, {64, 64, 4}, {192, 256, 4}, {96, 128, 4}, {64, 64, 4}, {256, 256, 4}, {128, 64, 4},
     {128, 64, 4},
 };
+// Two identifiers of earlier builds (a 256x256 tile with eight waves, a 128x128 tile with a 1x4 wave grid) never won
+// a shape against the kernels above in any sweep; their numbers stay reserved and a call that names one is refused.
+static bool variant_retired(int v) { return v == NEOGEMM_VARIANT_RETIRED_2 || v == NEOGEMM_VARIANT_RETIRED_8; }
 
 static bool is_aligned(const void* A, const void* B, const void* C, int64_t K, int64_t lda, int64_t ldb,
                        int64_t ldc) {
@@ -1938,7 +1937,7 @@ static const std::vector<PlanEntry>& plan_table() {
       PlanEntry e{field("M", -1), field("N", -1), field("K", -1), (int)field("b_layout", 0), (int)field("c_layout", 0),
                   (int)field("variant", -1), (int)field("split_k", 0)};
       if (e.M > 0 && e.N > 0 && e.K > 0 && e.variant > NEOGEMM_VARIANT_AUTO && e.variant < NEOGEMM_VARIANT_COUNT &&
-          e.split_k >= 1 && e.split_k <= 64 && (e.c_layout == NEOGEMM_C_ROW || e.c_layout == NEOGEMM_C_COL) &&
+          !variant_retired(e.variant) && e.split_k >= 1 && e.split_k <= 64 && (e.c_layout == NEOGEMM_C_ROW || e.c_layout == NEOGEMM_C_COL) &&
           (e.b_layout == NEOGEMM_B_KN || e.b_layout == NEOGEMM_B_NK))
         t.push_back(e);
       pos = end + 1;
@@ -2093,6 +2092,7 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
   if ((b_layout != NEOGEMM_B_KN && b_layout != NEOGEMM_B_NK) || (c_layout != NEOGEMM_C_ROW && c_layout != NEOGEMM_C_COL))
     return NEOGEMM_ERR_BAD_ARG;
   if (variant < 0 || variant >= NEOGEMM_VARIANT_COUNT || split_k < 0 || group_m < 0) return NEOGEMM_ERR_BAD_ARG;
+  if (variant_retired(variant)) return NEOGEMM_ERR_UNSUPPORTED;
   if (M == 0 || N == 0) return NEOGEMM_OK;
   if (!C || (K > 0 && (!A || !B))) return NEOGEMM_ERR_BAD_ARG;
   if (lda < K || ldb < (b_layout == NEOGEMM_B_KN ? N : K) || ldc < (c_layout == NEOGEMM_C_ROW ? N : M))
@@ -2275,13 +2275,11 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
 
   hipError_t e;
   switch (v) {
-    case NEOGEMM_VARIANT_T256x256_W8: e = launch_tile<256, 256, 2, 4>(a, ak, bk, st); break;
     case NEOGEMM_VARIANT_T256x256_W4: e = launch_tile<256, 256, 2, 2>(a, ak, bk, st); break;
     case NEOGEMM_VARIANT_T128x128_W4: e = launch_tile<128, 128, 2, 2>(a, ak, bk, st); break;
     case NEOGEMM_VARIANT_T256x128_W4: e = launch_tile<256, 128, 2, 2>(a, ak, bk, st); break;
     case NEOGEMM_VARIANT_T128x256_W4: e = launch_tile<128, 256, 2, 2>(a, ak, bk, st); break;
     case NEOGEMM_VARIANT_T64x128_W4: e = launch_tile<64, 128, 1, 4>(a, ak, bk, st); break;
-    case NEOGEMM_VARIANT_T128x128_W4S: e = launch_tile<128, 128, 1, 4>(a, ak, bk, st); break;
     case NEOGEMM_VARIANT_T192x256_W4: e = launch_tile<192, 256, 2, 2>(a, ak, bk, st); break;
     case NEOGEMM_VARIANT_T96x128_W4: e = launch_tile<96, 128, 2, 2>(a, ak, bk, st); break;
     case NEOGEMM_VARIANT_T64x64_W4: e = launch_tile<64, 64, 2, 2>(a, ak, bk, st); break;
@@ -2394,7 +2392,7 @@ int neogemm_bf16_profile(const void* A, const void* B, void* C, int64_t M, int64
                          int64_t ldb, int64_t ldc, int b_layout, void* hip_stream, int variant, int group_m,
                          unsigned long long* phase_cycles, size_t phase_cycles_bytes) {
   if (!phase_cycles) return NEOGEMM_ERR_BAD_ARG;
-  if (variant != NEOGEMM_VARIANT_T256x256_W8 && variant != NEOGEMM_VARIANT_T256x256_W4) return NEOGEMM_ERR_UNSUPPORTED;
+  if (variant != NEOGEMM_VARIANT_T256x256_W4) return NEOGEMM_ERR_UNSUPPORTED;
   if (phase_cycles_bytes < neogemm_bf16_profile_bytes(M, N, variant)) return NEOGEMM_ERR_WORKSPACE;
   return neogemm::run(A, B, C, M, N, K, lda, ldb, ldc, b_layout, NEOGEMM_C_ROW, nullptr, 0, hip_stream, variant, 1,
                       group_m, phase_cycles);
@@ -2402,8 +2400,8 @@ int neogemm_bf16_profile(const void* A, const void* B, void* C, int64_t M, int64
 
 size_t neogemm_bf16_profile_bytes(int64_t M, int64_t N, int variant) {
   if (M <= 0 || N <= 0) return 0;
-  const int waves = variant == NEOGEMM_VARIANT_T256x256_W4 ? 4 : 8;
-  return (size_t)neogemm::ceil_div(M, 256) * neogemm::ceil_div(N, 256) * waves * 4 * sizeof(unsigned long long);
+  if (variant != NEOGEMM_VARIANT_T256x256_W4) return 0;
+  return (size_t)neogemm::ceil_div(M, 256) * neogemm::ceil_div(N, 256) * 4 * 4 * sizeof(unsigned long long);
 }
 
 size_t neogemm_bf16_workspace_bytes(int64_t M, int64_t N, int64_t K) {

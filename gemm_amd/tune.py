@@ -21,7 +21,7 @@ import torch
 from . import _abi, gemm_into, plan
 from ._abi import B_KN, B_NK, C_COL, C_ROW, ERR_UNSUPPORTED, NeoGemmError
 
-CANDIDATE_VARIANTS = (_abi.VARIANT_T256x256_W4, _abi.VARIANT_C256x256_W4, _abi.VARIANT_T256x256_W8, _abi.VARIANT_T128x256_W4,
+CANDIDATE_VARIANTS = (_abi.VARIANT_T256x256_W4, _abi.VARIANT_C256x256_W4, _abi.VARIANT_T128x256_W4,
                       _abi.VARIANT_T256x128_W4, _abi.VARIANT_T128x128_W4, _abi.VARIANT_T64x128_W4,
                       _abi.VARIANT_T192x256_W4, _abi.VARIANT_T96x128_W4, _abi.VARIANT_T64x64_W4, _abi.VARIANT_SKINNY16, _abi.VARIANT_SKINNY32, _abi.VARIANT_SKINNY64,
                       _abi.VARIANT_SKINNY128, _abi.VARIANT_STRIP)

@@ -44,13 +44,13 @@ extern "C" {
 #define NEOGEMM_VARIANT_AUTO 0
 #define NEOGEMM_VARIANT_GENERIC 1   /* scalar-load fallback: any shape, stride, alignment */
 /* Tile variants: BM x BN macro-tile per workgroup, K in steps of 64, 16x16x32 MFMA; (r x c) = wave grid. */
-#define NEOGEMM_VARIANT_T256x256_W8 2 /* 256x256, 8 wave64 (2x4) */
+#define NEOGEMM_VARIANT_RETIRED_2 2   /* was 256x256 with 8 wave64: never the fastest on any shape; calls naming it are refused */
 #define NEOGEMM_VARIANT_T256x256_W4 3 /* 256x256, 4 wave64 (2x2): the default for large shapes */
 #define NEOGEMM_VARIANT_T128x128_W4 4 /* 128x128, 4 wave64 (2x2) */
 #define NEOGEMM_VARIANT_T256x128_W4 5 /* 256x128, 4 wave64 (2x2) */
 #define NEOGEMM_VARIANT_T128x256_W4 6 /* 128x256, 4 wave64 (2x2) */
 #define NEOGEMM_VARIANT_T64x128_W4 7  /* 64x128, 4 wave64 (1x4) */
-#define NEOGEMM_VARIANT_T128x128_W4S 8 /* 128x128, 4 wave64 (1x4) */
+#define NEOGEMM_VARIANT_RETIRED_8 8   /* was 128x128 with a 1x4 wave grid: likewise */
 /* Skinny M (or, with B [N,K], skinny N): a strip of 64 columns and all of K per workgroup, no split-K (decode shapes). */
 #define NEOGEMM_VARIANT_SKINNY16 9  /* M <= 16 */
 #define NEOGEMM_VARIANT_SKINNY32 10 /* M <= 32 */
@@ -175,10 +175,10 @@ int neogemm_bf16_plan(int64_t M, int64_t N, int64_t K, int b_layout, int c_layou
                       int* variant, int* split_k);
 
 /*
- * Instrumented run of a 256x256 variant (row-major C, no split-K): besides computing C, every wave
- * writes four shader-clock cycle counts {whole kernel, waiting for its own global->LDS loads, waiting
- * at the workgroup barrier, epilogue} to phase_cycles[(workgroup * waves + wave) * 4 + i], with
- * waves = 8 or 4 by variant and workgroup = launch order.  This is the per-phase cycle buffer of the
+ * Instrumented run of NEOGEMM_VARIANT_T256x256_W4 (row-major C, no split-K): besides computing C, every
+ * wave writes four shader-clock cycle counts {whole kernel, waiting for its own global->LDS loads, waiting
+ * at the workgroup barrier, epilogue} to phase_cycles[(workgroup * 4 + wave) * 4 + i], workgroup = launch
+ * order; other variants are refused with NEOGEMM_ERR_UNSUPPORTED.  This is the per-phase cycle buffer of the
  * reference's harness (the `DB` array: cublass/matmul.cu:99-106 allocation, :149-165 decode), which
  * no kernel in the reference fills in.  phase_cycles is device memory of at least
  * neogemm_bf16_profile_bytes(M, N, variant) bytes.  The timers cost a few percent; never time with it.

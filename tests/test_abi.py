@@ -56,8 +56,8 @@ def test_plan_for_the_benchmark_configs():
         assert v == _abi.VARIANT_C256x256_W4 and s == 1   # K in whole periods of 128, A K-major: the chained kernel
         assert _abi.plan(n, n, n, _abi.B_NK, _abi.C_COL) == (_abi.VARIANT_C256x256_W4, 1)   # the reference's call
         # B [K,N] with a column-major C puts the MN-major operand on the rows, K = 8256 is not whole periods: slab kernel
-        assert _abi.plan(n, n, n, _abi.B_KN, _abi.C_COL)[0] in (_abi.VARIANT_T256x256_W4, _abi.VARIANT_T256x256_W8)
-        assert _abi.plan(n, n, n + 64)[0] in (_abi.VARIANT_T256x256_W4, _abi.VARIANT_T256x256_W8)
+        assert _abi.plan(n, n, n, _abi.B_KN, _abi.C_COL)[0] == _abi.VARIANT_T256x256_W4
+        assert _abi.plan(n, n, n + 64)[0] == _abi.VARIANT_T256x256_W4
     # shapes with few output tiles split K and need a workspace of split * M * N floats (skinny M with a row-major C
     # runs the streaming kernel instead, without split-K)
     for M, N, K in ((16, 14336, 4096), (64, 14336, 4096), (128, 14336, 4096), (1024, 1024, 32768), (512, 512, 512)):
@@ -153,7 +153,7 @@ def test_plan_rejects_null_outputs():
 
 def test_profile_bytes():
     lib = _abi.load()
-    assert lib.neogemm_bf16_profile_bytes(8192, 8192, _abi.VARIANT_T256x256_W8) == 1024 * 8 * 4 * 8
+    assert lib.neogemm_bf16_profile_bytes(8192, 8192, 2) == 0   # a retired variant number: nothing to profile
     assert lib.neogemm_bf16_profile_bytes(8192, 8192, _abi.VARIANT_T256x256_W4) == 1024 * 4 * 4 * 8
     assert lib.neogemm_bf16_profile_bytes(0, 8, _abi.VARIANT_T256x256_W4) == 0
 
@@ -167,7 +167,8 @@ def test_plan_table_overrides_the_model(tmp_path):
     table = tmp_path / "plan.json"
     table.write_text(json.dumps([
         {"M": 512, "N": 512, "K": 512, "c_layout": 0, "variant": _abi.VARIANT_T128x128_W4, "split_k": 2},
-        {"M": 4096, "N": 4096, "K": 4096, "variant": _abi.VARIANT_T256x256_W8, "split_k": 1},   # c_layout defaults to 0
+        {"M": 4096, "N": 4096, "K": 4096, "variant": _abi.VARIANT_T256x256_W4, "split_k": 1},   # c_layout defaults to 0
+        {"M": 3072, "N": 3072, "K": 3072, "c_layout": 0, "variant": 2, "split_k": 1},            # a retired variant number
         {"M": 8192, "N": 8192, "K": 8192, "c_layout": 0, "variant": 99, "split_k": 1},           # unknown variant
         {"M": 1024, "N": 1024, "K": 1024, "c_layout": 0, "variant": _abi.VARIANT_T128x128_W4, "split_k": 0},  # bad split
         {"M": 2048, "N": 2048, "K": 2048, "b_layout": 1, "c_layout": 1, "variant": _abi.VARIANT_T128x256_W4, "split_k": 1},
@@ -179,7 +180,7 @@ def test_plan_table_overrides_the_model(tmp_path):
     env = dict(os.environ, NEOGEMM_PLAN_TABLE=str(table))
     out = subprocess.run([sys.executable, "-c", code], env=env, cwd=ROOT, capture_output=True, text=True, check=True).stdout
     model = (_abi.plan(512, 512, 512), _abi.plan(8192, 8192, 8192), _abi.plan(1024, 1024, 1024))
-    want = ((_abi.VARIANT_T128x128_W4, 2), (_abi.VARIANT_T256x256_W8, 1), model[1], model[2],
+    want = ((_abi.VARIANT_T128x128_W4, 2), (_abi.VARIANT_T256x256_W4, 1), model[1], model[2],
             _abi.plan(512, 512, 512, c_layout=1), 2 * 512 * 512 * 4,
             # an entry is keyed on both layouts: B [N,K] calls of a shape tuned with B [K,N] keep the model's choice
             _abi.plan(512, 512, 512, b_layout=1), (_abi.VARIANT_T128x256_W4, 1), _abi.plan(2048, 2048, 2048, 0, 1))
@@ -204,7 +205,7 @@ def test_shipped_plan_table():
     assert len({r[:5] for r in rows}) == len(rows)                       # one entry per shape and layout pair
     tile_variants = (_abi.VARIANT_T256x256_W4, _abi.VARIANT_T128x128_W4, _abi.VARIANT_T256x128_W4, _abi.VARIANT_T128x256_W4,
                      _abi.VARIANT_T64x128_W4, _abi.VARIANT_T192x256_W4, _abi.VARIANT_T96x128_W4, _abi.VARIANT_T64x64_W4,
-                     _abi.VARIANT_C256x256_W4, _abi.VARIANT_T256x256_W8)
+                     _abi.VARIANT_C256x256_W4)
     for (M, N, K, b, c, v, s) in rows:
         assert b in (0, 1) and c in (0, 1) and 1 <= s <= 64 and s * 128 <= K
         assert v in tile_variants + (_abi.VARIANT_SKINNY16, _abi.VARIANT_SKINNY32, _abi.VARIANT_SKINNY64, _abi.VARIANT_SKINNY128,

@@ -21,15 +21,15 @@ from oracle import gemm_oracle as o
 
 pytestmark = pytest.mark.gpu
 
-TILE_VARIANTS = [g.VARIANT_T256x256_W8, g.VARIANT_T256x256_W4, g.VARIANT_T128x128_W4, g.VARIANT_T256x128_W4,
-                 g.VARIANT_T128x256_W4, g.VARIANT_T64x128_W4, g.VARIANT_T128x128_W4S, g.VARIANT_T192x256_W4,
+TILE_VARIANTS = [g.VARIANT_T256x256_W4, g.VARIANT_T128x128_W4, g.VARIANT_T256x128_W4,
+                 g.VARIANT_T128x256_W4, g.VARIANT_T64x128_W4, g.VARIANT_T192x256_W4,
                  g.VARIANT_T96x128_W4, g.VARIANT_T64x64_W4]
 ALL_VARIANTS = [g.VARIANT_GENERIC] + TILE_VARIANTS
 
 
-TILE_SHAPE = {g.VARIANT_T256x256_W8: (256, 256), g.VARIANT_T256x256_W4: (256, 256), g.VARIANT_T128x128_W4: (128, 128),
+TILE_SHAPE = {g.VARIANT_T256x256_W4: (256, 256), g.VARIANT_T128x128_W4: (128, 128),
               g.VARIANT_T256x128_W4: (256, 128), g.VARIANT_T128x256_W4: (128, 256), g.VARIANT_T64x128_W4: (64, 128),
-              g.VARIANT_T128x128_W4S: (128, 128), g.VARIANT_T192x256_W4: (192, 256), g.VARIANT_T96x128_W4: (96, 128),
+              g.VARIANT_T192x256_W4: (192, 256), g.VARIANT_T96x128_W4: (96, 128),
               g.VARIANT_T64x64_W4: (64, 64)}
 
 
@@ -275,7 +275,7 @@ def test_ragged_shapes_forced_tile_kernels(dev, variant, M, N, K):
 # The tile kernels stage K in 64-deep tiles / 32-deep slabs with a prologue, a steady loop that is entered
 # from seven K tiles on and unrolls two periods, and a tail: every K below walks a different way through
 # them (tile counts 1..13, with and without a partial last tile), once per operand combination.
-@pytest.mark.parametrize("variant", [g.VARIANT_T256x256_W4, g.VARIANT_T256x256_W8, g.VARIANT_T128x128_W4, g.VARIANT_T96x128_W4,
+@pytest.mark.parametrize("variant", [g.VARIANT_T256x256_W4, g.VARIANT_T128x128_W4, g.VARIANT_T96x128_W4,
                                      g.VARIANT_T64x64_W4])
 @pytest.mark.parametrize("b_layout,c_layout", [(g.B_KN, g.C_ROW), (g.B_NK, g.C_ROW), (g.B_KN, g.C_COL)])
 def test_k_loop_transitions(dev, variant, b_layout, c_layout):
@@ -602,7 +602,7 @@ def test_profile_entry_point(dev):
     A, B = o.make_inputs(M, N, K, seed=12)
     Ad, Bd = A.to(dev), B.to(dev)
     C = torch.zeros(M, N, dtype=torch.bfloat16, device=dev)
-    for variant, waves in ((g.VARIANT_T256x256_W8, 8), (g.VARIANT_T256x256_W4, 4)):
+    for variant, waves in ((g.VARIANT_T256x256_W4, 4),):
         nb = lib.neogemm_bf16_profile_bytes(M, N, variant)
         buf = torch.zeros(nb // 8, dtype=torch.int64, device=dev)
         st = lib.neogemm_bf16_profile(Ad.data_ptr(), Bd.data_ptr(), C.data_ptr(), M, N, K, K, N, N, 0, None, variant, 0,
@@ -615,6 +615,13 @@ def test_profile_entry_point(dev):
         o.assert_parity(C, A, B, what="profiled run")
         assert lib.neogemm_bf16_profile(Ad.data_ptr(), Bd.data_ptr(), C.data_ptr(), M, N, K, K, N, N, 0, None, variant, 0,
                                         buf.data_ptr(), 8) == _abi.ERR_WORKSPACE
+    # the instrumented build exists for that one kernel; retired variant numbers are refused everywhere
+    for variant in (2, 8, g.VARIANT_T128x128_W4):
+        assert lib.neogemm_bf16_profile(Ad.data_ptr(), Bd.data_ptr(), C.data_ptr(), M, N, K, K, N, N, 0, None, variant, 0,
+                                        buf.data_ptr(), nb) == _abi.ERR_UNSUPPORTED
+    for variant in (2, 8):
+        with pytest.raises(g.NeoGemmError):
+            g.gemm_into(Ad, Bd, C, M, N, K, K, N, N, g.B_KN, g.C_ROW, variant)
 
 
 def test_benchmark_driver(dev):
