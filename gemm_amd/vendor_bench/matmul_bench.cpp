@@ -9,7 +9,7 @@
 //
 //   matmul_bench M N K [reps=100] [b_layout=0|1] [variant=0] [split_k=0] [group_m=0] [nbuf=1]
 //   matmul_bench ceiling [preheat_ms=1000]
-//   matmul_bench loadpath M N K [b_layout=1] [strip=64]
+//   matmul_bench loadpath M N K [b_layout=1] [strip=64] [row_tiles=1] [wide=0] [k_parts=1]
 //
 // One line of JSON per library on stdout.  Lines of timed runs carry "t0" / "t1", CLOCK_MONOTONIC seconds around the
 // timed batches, so that a parent process that samples the board's power and clocks can tell which samples belong to
@@ -488,34 +488,55 @@ static int run_ceiling(int preheat_ms) {
 
 // ---- load path of a decode-shaped GEMM, arithmetic taken away ---------------------------------------
 // One 128-deep step of a workgroup: B 2 * strip / 8 requests (8 rows x 128 B each; B [K,N]: 16 requests of 8 k-rows x
-// 128 B), A 2 * M / 8 requests.  The NW waves take the requests of a step round-robin; each keeps at most D in flight.
+// 128 B per 64 columns), A 2 * rows / 8 requests.  The NW waves take the requests of a step round-robin; each keeps at
+// most D in flight.  With row_tiles > 1 a strip belongs to that many workgroups, each with its share of A's rows (the
+// decomposition of a stream-K library kernel with a 64-row tile: B is requested row_tiles times, once from HBM).
 typedef __attribute__((ext_vector_type(4))) int ci32x4b;
 template <int D>
 __global__ __launch_bounds__(512) void loadpath_kernel(const char* A, const char* B, float* out, int M, int K, int N, int strip,
-                                                       int with_a, int b_kn) {
+                                                       int with_a, int b_kn, int row_tiles, int wide, int k_parts) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   const uint32_t l0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), nw = blockDim.x >> 6;
   const int lane = threadIdx.x & 63;
   // one buffer resource per operand; a request is told apart by a scalar offset.  Lanes past the end of A (rows beyond
   // M) are out of the resource's range: they read as zeros and touch no memory.
-  const uint64_t bb = b_kn ? (uint64_t)B + (uint64_t)blockIdx.x * strip * 2 : (uint64_t)B + (uint64_t)blockIdx.x * strip * K * 2;
+  // the workgroups of one strip sit on one XCD (workgroup id mod 8), next to each other in dispatch order, so that the
+  // strip's B comes out of HBM once and out of that XCD's L2 for the others; the host rounds the strip count to eights
+  // With k_parts > 1 (and row_tiles 1) a strip belongs to that many workgroups, each with its range of K (a split-K or
+  // stream-K decomposition: B is requested once, A's bytes per workgroup shrink); part p of every strip runs on the
+  // XCDs p, p + k_parts, ..., so an XCD's L2 holds one range of A.
+  const int kp = k_parts > 1 ? (blockIdx.x & 7) % k_parts : 0;
+  const int rt = k_parts > 1 ? 0 : (blockIdx.x >> 3) % row_tiles;
+  const int strip_id = k_parts > 1 ? (blockIdx.x >> 3) * (8 / k_parts) + (blockIdx.x & 7) / k_parts
+                                   : (blockIdx.x / (8 * row_tiles)) * 8 + (blockIdx.x & 7);
+  const int tile_rows = (M + row_tiles - 1) / row_tiles;
+  const int rows = min(tile_rows, M - rt * tile_rows);   // the host checked that every tile has rows
+  const uint64_t bb = b_kn ? (uint64_t)B + (uint64_t)strip_id * strip * 2 : (uint64_t)B + (uint64_t)strip_id * strip * K * 2;
+  const uint64_t ab = (uint64_t)A + (uint64_t)rt * tile_rows * K * 2;
   const uint32_t ldb = b_kn ? (uint32_t)N * 2 : (uint32_t)K * 2;
-  const ci32x4b ra = {(int)(uint32_t)(uint64_t)A, (int)(((uint64_t)A >> 32) & 0xffff), (int)((uint32_t)M * K * 2), 0x00020000};
-  const uint32_t voff_b = (lane >> 3) * ldb + (lane & 7) * 16, voff_a = (lane >> 3) * (uint32_t)K * 2 + (lane & 7) * 16;
+  const ci32x4b ra = {(int)(uint32_t)ab, (int)((ab >> 32) & 0xffff), (int)((uint32_t)rows * K * 2), 0x00020000};
+  // a request is 8 rows x 128 bytes, or (wide) 4 rows x 256 bytes: the same eight cache lines, in half as many rows
+  // (wide: bit 0 for A's requests, bit 1 for B's)
+  const bool wide_a = wide & 1, wide_b = wide & 2;
+  const uint32_t voff_b = wide_b ? (lane >> 4) * ldb + (lane & 15) * 16 : (lane >> 3) * ldb + (lane & 7) * 16;
+  const uint32_t voff_a = wide_a ? (lane >> 4) * (uint32_t)K * 2 + (lane & 15) * 16 : (lane >> 3) * (uint32_t)K * 2 + (lane & 7) * 16;
   asm volatile("s_mov_b32 m0, %0" ::"s"(l0 + wave * 1024) : "memory");
-  const int nb = b_kn ? 16 : strip / 8 * 2, na = with_a ? (M + 7) / 8 * 2 : 0;
-  for (int s = 0; s < K / 128; ++s) {
+  const int halves = strip / 64;   // B [K,N]: 128-byte pieces of a k-row
+  const int nb = b_kn ? 16 * halves : strip / 8 * 2, na = with_a ? (rows + 7) / 8 * 2 : 0;
+  const int steps = K / 128 / k_parts;
+  for (int s = kp * steps; s < (kp + 1) * steps; ++s) {
     // B [N,K]: the strip's rows, 256 bytes further along K per step; B [K,N]: 128 k-rows further down per step
     const uint64_t bs = b_kn ? bb + (uint64_t)s * 128 * ldb : bb + (uint64_t)s * 256;
     const ci32x4b rb = {(int)(uint32_t)bs, (int)((bs >> 32) & 0xffff), (int)0x7fffffff, 0x00020000};
     for (int r = wave; r < nb + na; r += nw) {
       if (r < nb) {
-        const uint32_t soff = b_kn ? (uint32_t)r * 8 * ldb : (uint32_t)(r >> 1) * 8 * ldb + (r & 1) * 128;
+        const uint32_t soff = wide_b ? (uint32_t)r * 4 * ldb   // B [K,N]: the host asked for a strip of 128 columns
+                              : b_kn ? (uint32_t)(r / halves) * 8 * ldb + (r % halves) * 128 : (uint32_t)(r >> 1) * 8 * ldb + (r & 1) * 128;
         asm volatile("buffer_load_dwordx4 %0, %1, %2 offen sc1 lds" ::"v"(voff_b), "s"(rb), "s"(soff) : "memory");
       } else {
         const int q = r - nb;
-        const uint32_t soff = (uint32_t)(q >> 1) * 8 * K * 2 + (q & 1) * 128 + (uint32_t)s * 256;
+        const uint32_t soff = wide_a ? (uint32_t)q * 4 * K * 2 + (uint32_t)s * 256 : (uint32_t)(q >> 1) * 8 * K * 2 + (q & 1) * 128 + (uint32_t)s * 256;
         asm volatile("buffer_load_dwordx4 %0, %1, %2 offen sc1 lds" ::"v"(voff_a), "s"(ra), "s"(soff) : "memory");
       }
       asm volatile("s_waitcnt vmcnt(%0)" ::"n"(D) : "memory");
@@ -525,9 +546,14 @@ __global__ __launch_bounds__(512) void loadpath_kernel(const char* A, const char
   out[blockIdx.x * blockDim.x + threadIdx.x] = ((float*)smem)[threadIdx.x];
 }
 
-static int run_loadpath(int64_t M, int64_t N, int64_t K, int b_layout, int strip) {
-  if (M < 1 || N < strip || K < 128 || K % 128 || N % strip || strip % 8 || strip > 64 || (b_layout == 0 && strip != 64)) {
-    fprintf(stderr, "loadpath: K a multiple of 128, N a multiple of the strip (a multiple of 8 up to 64; 64 with B [K,N])\n");
+static int run_loadpath(int64_t M, int64_t N, int64_t K, int b_layout, int strip, int row_tiles, int wide, int k_parts) {
+  if (M < 1 || N < strip || K < 128 || K % 128 || N % strip || strip % 8 || strip < 8 || strip > 128 || (b_layout == 0 && strip % 64) ||
+      (k_parts != 1 && k_parts != 2 && k_parts != 4 && k_parts != 8) || (k_parts > 1 && (row_tiles != 1 || (N / strip) % (8 / k_parts) ||
+                                                                                    K / 128 % k_parts)) ||
+      wide < 0 || wide > 3 || ((wide & 2) && b_layout == 0 && strip != 128) || ((wide & 2) && strip % 4) || row_tiles < 1 || (row_tiles > 1 && (N / strip) % 8) || (M + row_tiles - 1) / row_tiles * (row_tiles - 1) >= M || (uint64_t)M * K * 2 > 0x7fffffffull ||
+      (uint64_t)strip * K * 2 > 0x7fffffffull || (uint64_t)K * N * 2 > 0x7fffffffull * 2) {
+    fprintf(stderr, "loadpath: K a multiple of 128, N a multiple of the strip (a multiple of 8 up to 128; 64 or 128 with B [K,N]), "
+                    "row_tiles >= 1 with rows in every tile (and then a strip count that is a multiple of 8)\n");
     return 2;
   }
   hipStream_t st;
@@ -542,21 +568,22 @@ static int run_loadpath(int64_t M, int64_t N, int64_t K, int b_layout, int strip
     HIP_OK(hipMalloc(&p, b_bytes));
     HIP_OK(hipMemset(p, 1, b_bytes));
   }
-  const int wgs = (int)(N / strip);
+  const int wgs = (int)(N / strip) * row_tiles * k_parts;
   HIP_OK(hipMalloc(&dout, (size_t)wgs * 512 * 4));
   HIP_OK(hipFuncSetAttribute((const void*)loadpath_kernel<16>, hipFuncAttributeMaxDynamicSharedMemorySize, 65536));
   for (int with_a = 0; with_a < 2; ++with_a)
     for (int threads : {256, 512}) {
       auto launch = [&](int i) {
         loadpath_kernel<16><<<wgs, threads, 65536, st>>>((const char*)dA, (const char*)dB[i % nbuf], (float*)dout, (int)M, (int)K, (int)N, strip,
-                                                         with_a, b_layout == 0);
+                                                         with_a, b_layout == 0, row_tiles, wide, k_parts);
       };
       const double ms = time_ms(launch, 100, st);
       HIP_OK(hipGetLastError());
-      printf("{\"loadpath\": \"%s\", \"M\": %lld, \"N\": %lld, \"K\": %lld, \"b_layout\": %d, \"strip\": %d, \"workgroups\": %d, "
+      printf("{\"loadpath\": \"%s\", \"M\": %lld, \"N\": %lld, \"K\": %lld, \"b_layout\": %d, \"strip\": %d, \"row_tiles\": %d, \"k_parts\": %d, \"request\": \"%s\", \"workgroups\": %d, "
              "\"waves\": %d, \"requests_in_flight_per_wave\": 16, \"us\": %.2f, \"b_tbps\": %.2f, \"a_from_l2_mb\": %.1f}\n",
              with_a ? "B from HBM + all of A from L2 per workgroup" : "B from HBM only", (long long)M, (long long)N, (long long)K,
-             b_layout, strip, wgs, threads / 64, ms * 1e3, (double)b_bytes / ms / 1e9, with_a ? (double)wgs * M * K * 2 / 1e6 : 0.0);
+             b_layout, strip, row_tiles, k_parts, wide == 3 ? "4 rows x 256 B" : wide == 1 ? "A 4 rows x 256 B, B 8 rows x 128 B" : wide == 2 ? "A 8 rows x 128 B, B 4 rows x 256 B" : "8 rows x 128 B", wgs, threads / 64, ms * 1e3, (double)b_bytes / ms / 1e9,
+             with_a ? (double)(N / strip) * M * K * 2 / 1e6 : 0.0);   // (each of k_parts workgroups takes its share of these)
       fflush(stdout);
     }
   return 0;
@@ -565,10 +592,12 @@ static int run_loadpath(int64_t M, int64_t N, int64_t K, int b_layout, int strip
 int main(int argc, char** argv) {
   if (argc >= 2 && strcmp(argv[1], "ceiling") == 0) return run_ceiling(argc > 2 ? atoi(argv[2]) : 1000);
   if (argc >= 5 && strcmp(argv[1], "loadpath") == 0)
-    return run_loadpath(atoll(argv[2]), atoll(argv[3]), atoll(argv[4]), argc > 5 ? atoi(argv[5]) : 1, argc > 6 ? atoi(argv[6]) : 64);
+    return run_loadpath(atoll(argv[2]), atoll(argv[3]), atoll(argv[4]), argc > 5 ? atoi(argv[5]) : 1, argc > 6 ? atoi(argv[6]) : 64,
+                        argc > 7 ? atoi(argv[7]) : 1, argc > 8 ? atoi(argv[8]) : 0,
+                        argc > 9 ? atoi(argv[9]) : 1);
   if (argc < 4) {
     fprintf(stderr, "usage: %s M N K [reps] [b_layout] [variant] [split_k] [group_m] [nbuf]\n       %s ceiling [preheat_ms]\n"
-            "       %s loadpath M N K [b_layout] [strip]\n", argv[0], argv[0], argv[0]);
+            "       %s loadpath M N K [b_layout] [strip] [row_tiles] [wide] [k_parts]\n", argv[0], argv[0], argv[0]);
     return 2;
   }
   const int64_t M = atoll(argv[1]), N = atoll(argv[2]), K = atoll(argv[3]);
