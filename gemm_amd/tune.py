@@ -119,6 +119,9 @@ def main():
     ap.add_argument("--inc", help="with --merge: write the merged table as the library's default-plan include file")
     ap.add_argument("--margin", type=float, default=0.03, help="minimum relative gain over the model's choice")
     ap.add_argument("--nbuf", type=int, default=1, help="rotate this many B buffers (streaming shapes)")
+    ap.add_argument("--cold-weights-mb", type=float, default=0.0,
+                    help="rotate as many B buffers as it takes to exceed this many MB (more than the last-level cache: every "
+                         "launch then streams its B from HBM, as a layer's weights are in inference); overrides --nbuf")
     ap.add_argument("--b-layout", type=int, default=B_KN, choices=(B_KN, B_NK), help="0: B [K,N], 1: B [N,K]")
     ap.add_argument("--c-layout", type=int, default=C_ROW, choices=(C_ROW, C_COL), help="0: row-major C, 1: column-major")
     args = ap.parse_args()
@@ -138,7 +141,10 @@ def main():
     table = []
     for sh in args.shapes:
         M, N, K = (int(x) for x in sh.lower().split("x"))
-        model, t_model, best, t_best = tune_shape(M, N, K, args.nbuf, b_layout=args.b_layout, c_layout=args.c_layout)
+        nbuf = args.nbuf
+        if args.cold_weights_mb > 0:
+            nbuf = max(2, min(32, int(args.cold_weights_mb * 1e6 // (2.0 * N * K)) + 1))
+        model, t_model, best, t_best = tune_shape(M, N, K, nbuf, b_layout=args.b_layout, c_layout=args.c_layout)
         if best != model and t_best < t_model * (1.0 - args.margin):
             table.append({"M": M, "N": N, "K": K, "b_layout": args.b_layout, "c_layout": args.c_layout,
                           "variant": best[0], "split_k": best[1]})
