@@ -9,7 +9,7 @@
 //
 //   matmul_bench M N K [reps=100] [b_layout=0|1] [variant=0] [split_k=0] [group_m=0] [nbuf=1]
 //   matmul_bench ceiling [preheat_ms=1000]
-//   matmul_bench loadpath M N K [b_layout=1] [strip=64] [row_tiles=1] [wide=0] [k_parts=1]
+//   matmul_bench loadpath M N K [b_layout=1] [strip=64] [row_tiles=1] [wide=0] [k_parts=1] [step_depth=128]
 //
 // One line of JSON per library on stdout.  Lines of timed runs carry "t0" / "t1", CLOCK_MONOTONIC seconds around the
 // timed batches, so that a parent process that samples the board's power and clocks can tell which samples belong to
@@ -494,7 +494,7 @@ static int run_ceiling(int preheat_ms) {
 typedef __attribute__((ext_vector_type(4))) int ci32x4b;
 template <int D>
 __global__ __launch_bounds__(512) void loadpath_kernel(const char* A, const char* B, float* out, int M, int K, int N, int strip,
-                                                       int with_a, int b_kn, int row_tiles, int wide, int k_parts) {
+                                                       int with_a, int b_kn, int row_tiles, int wide, int k_parts, int pshift) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   const uint32_t l0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), nw = blockDim.x >> 6;
@@ -523,20 +523,23 @@ __global__ __launch_bounds__(512) void loadpath_kernel(const char* A, const char
   const uint32_t voff_a = wide_a ? (lane >> 4) * (uint32_t)K * 2 + (lane & 15) * 16 : (lane >> 3) * (uint32_t)K * 2 + (lane & 7) * 16;
   asm volatile("s_mov_b32 m0, %0" ::"s"(l0 + wave * 1024) : "memory");
   const int halves = strip / 64;   // B [K,N]: 128-byte pieces of a k-row
-  const int nb = b_kn ? 16 * halves : strip / 8 * 2, na = with_a ? (rows + 7) / 8 * 2 : 0;
-  const int steps = K / 128 / k_parts;
+  // K-major operands: a step is 64 << pshift deep (pshift 1: 128), i.e. 1 << pshift pieces of 128 bytes per row, requested
+  // back to back; the deeper the step, the longer the run of consecutive bytes a row contributes at a time
+  const int pieces = 1 << pshift;
+  const int nb = b_kn ? 16 * halves : strip / 8 * pieces, na = with_a ? (rows + 7) / 8 * pieces : 0;
+  const int steps = b_kn ? K / 128 / k_parts : K / (64 << pshift) / k_parts;
   for (int s = kp * steps; s < (kp + 1) * steps; ++s) {
     // B [N,K]: the strip's rows, 256 bytes further along K per step; B [K,N]: 128 k-rows further down per step
-    const uint64_t bs = b_kn ? bb + (uint64_t)s * 128 * ldb : bb + (uint64_t)s * 256;
+    const uint64_t bs = b_kn ? bb + (uint64_t)s * 128 * ldb : bb + (uint64_t)s * (128u << pshift);
     const ci32x4b rb = {(int)(uint32_t)bs, (int)((bs >> 32) & 0xffff), (int)0x7fffffff, 0x00020000};
     for (int r = wave; r < nb + na; r += nw) {
       if (r < nb) {
         const uint32_t soff = wide_b ? (uint32_t)r * 4 * ldb   // B [K,N]: the host asked for a strip of 128 columns
-                              : b_kn ? (uint32_t)(r / halves) * 8 * ldb + (r % halves) * 128 : (uint32_t)(r >> 1) * 8 * ldb + (r & 1) * 128;
+                              : b_kn ? (uint32_t)(r / halves) * 8 * ldb + (r % halves) * 128 : (uint32_t)(r >> pshift) * 8 * ldb + (r & (pieces - 1)) * 128;
         asm volatile("buffer_load_dwordx4 %0, %1, %2 offen sc1 lds" ::"v"(voff_b), "s"(rb), "s"(soff) : "memory");
       } else {
         const int q = r - nb;
-        const uint32_t soff = wide_a ? (uint32_t)q * 4 * K * 2 + (uint32_t)s * 256 : (uint32_t)(q >> 1) * 8 * K * 2 + (q & 1) * 128 + (uint32_t)s * 256;
+        const uint32_t soff = wide_a ? (uint32_t)q * 4 * K * 2 + (uint32_t)s * 256 : (uint32_t)(q >> pshift) * 8 * K * 2 + (q & (pieces - 1)) * 128 + (uint32_t)s * (b_kn ? 256u : 128u << pshift);
         asm volatile("buffer_load_dwordx4 %0, %1, %2 offen sc1 lds" ::"v"(voff_a), "s"(ra), "s"(soff) : "memory");
       }
       asm volatile("s_waitcnt vmcnt(%0)" ::"n"(D) : "memory");
@@ -546,11 +549,12 @@ __global__ __launch_bounds__(512) void loadpath_kernel(const char* A, const char
   out[blockIdx.x * blockDim.x + threadIdx.x] = ((float*)smem)[threadIdx.x];
 }
 
-static int run_loadpath(int64_t M, int64_t N, int64_t K, int b_layout, int strip, int row_tiles, int wide, int k_parts) {
+static int run_loadpath(int64_t M, int64_t N, int64_t K, int b_layout, int strip, int row_tiles, int wide, int k_parts, int depth) {
   if (M < 1 || N < strip || K < 128 || K % 128 || N % strip || strip % 8 || strip < 8 || strip > 128 || (b_layout == 0 && strip % 64) ||
       (k_parts != 1 && k_parts != 2 && k_parts != 4 && k_parts != 8) || (k_parts > 1 && (row_tiles != 1 || (N / strip) % (8 / k_parts) ||
                                                                                     K / 128 % k_parts)) ||
-      wide < 0 || wide > 3 || ((wide & 2) && b_layout == 0 && strip != 128) || ((wide & 2) && strip % 4) || row_tiles < 1 || (row_tiles > 1 && (N / strip) % 8) || (M + row_tiles - 1) / row_tiles * (row_tiles - 1) >= M || (uint64_t)M * K * 2 > 0x7fffffffull ||
+      (depth != 128 && depth != 256 && depth != 512 && depth != 1024) || (depth != 128 && (b_layout == 0 || wide)) ||
+      K % (depth * k_parts) || wide < 0 || wide > 3 || ((wide & 2) && b_layout == 0 && strip != 128) || ((wide & 2) && strip % 4) || row_tiles < 1 || (row_tiles > 1 && (N / strip) % 8) || (M + row_tiles - 1) / row_tiles * (row_tiles - 1) >= M || (uint64_t)M * K * 2 > 0x7fffffffull ||
       (uint64_t)strip * K * 2 > 0x7fffffffull || (uint64_t)K * N * 2 > 0x7fffffffull * 2) {
     fprintf(stderr, "loadpath: K a multiple of 128, N a multiple of the strip (a multiple of 8 up to 128; 64 or 128 with B [K,N]), "
                     "row_tiles >= 1 with rows in every tile (and then a strip count that is a multiple of 8)\n");
@@ -575,14 +579,14 @@ static int run_loadpath(int64_t M, int64_t N, int64_t K, int b_layout, int strip
     for (int threads : {256, 512}) {
       auto launch = [&](int i) {
         loadpath_kernel<16><<<wgs, threads, 65536, st>>>((const char*)dA, (const char*)dB[i % nbuf], (float*)dout, (int)M, (int)K, (int)N, strip,
-                                                         with_a, b_layout == 0, row_tiles, wide, k_parts);
+                                                         with_a, b_layout == 0, row_tiles, wide, k_parts, depth == 1024 ? 4 : depth == 512 ? 3 : depth == 256 ? 2 : 1);
       };
       const double ms = time_ms(launch, 100, st);
       HIP_OK(hipGetLastError());
-      printf("{\"loadpath\": \"%s\", \"M\": %lld, \"N\": %lld, \"K\": %lld, \"b_layout\": %d, \"strip\": %d, \"row_tiles\": %d, \"k_parts\": %d, \"request\": \"%s\", \"workgroups\": %d, "
+      printf("{\"loadpath\": \"%s\", \"M\": %lld, \"N\": %lld, \"K\": %lld, \"b_layout\": %d, \"strip\": %d, \"row_tiles\": %d, \"k_parts\": %d, \"step_depth\": %d, \"request\": \"%s\", \"workgroups\": %d, "
              "\"waves\": %d, \"requests_in_flight_per_wave\": 16, \"us\": %.2f, \"b_tbps\": %.2f, \"a_from_l2_mb\": %.1f}\n",
              with_a ? "B from HBM + all of A from L2 per workgroup" : "B from HBM only", (long long)M, (long long)N, (long long)K,
-             b_layout, strip, row_tiles, k_parts, wide == 3 ? "4 rows x 256 B" : wide == 1 ? "A 4 rows x 256 B, B 8 rows x 128 B" : wide == 2 ? "A 8 rows x 128 B, B 4 rows x 256 B" : "8 rows x 128 B", wgs, threads / 64, ms * 1e3, (double)b_bytes / ms / 1e9,
+             b_layout, strip, row_tiles, k_parts, depth, wide == 3 ? "4 rows x 256 B" : wide == 1 ? "A 4 rows x 256 B, B 8 rows x 128 B" : wide == 2 ? "A 8 rows x 128 B, B 4 rows x 256 B" : "8 rows x 128 B", wgs, threads / 64, ms * 1e3, (double)b_bytes / ms / 1e9,
              with_a ? (double)(N / strip) * M * K * 2 / 1e6 : 0.0);   // (each of k_parts workgroups takes its share of these)
       fflush(stdout);
     }
@@ -594,10 +598,10 @@ int main(int argc, char** argv) {
   if (argc >= 5 && strcmp(argv[1], "loadpath") == 0)
     return run_loadpath(atoll(argv[2]), atoll(argv[3]), atoll(argv[4]), argc > 5 ? atoi(argv[5]) : 1, argc > 6 ? atoi(argv[6]) : 64,
                         argc > 7 ? atoi(argv[7]) : 1, argc > 8 ? atoi(argv[8]) : 0,
-                        argc > 9 ? atoi(argv[9]) : 1);
+                        argc > 9 ? atoi(argv[9]) : 1, argc > 10 ? atoi(argv[10]) : 128);
   if (argc < 4) {
     fprintf(stderr, "usage: %s M N K [reps] [b_layout] [variant] [split_k] [group_m] [nbuf]\n       %s ceiling [preheat_ms]\n"
-            "       %s loadpath M N K [b_layout] [strip] [row_tiles] [wide] [k_parts]\n", argv[0], argv[0], argv[0]);
+            "       %s loadpath M N K [b_layout] [strip] [row_tiles] [wide] [k_parts] [step_depth]\n", argv[0], argv[0], argv[0]);
     return 2;
   }
   const int64_t M = atoll(argv[1]), N = atoll(argv[2]), K = atoll(argv[3]);
