@@ -1034,3 +1034,23 @@ def test_skinny_n_runs_the_transposed_problem(dev):
         A, Bkn = o.make_inputs(512, cols, 256, seed=1)
         with pytest.raises(g.NeoGemmError):
             run_abi(A, Bkn, dev, g.B_KN, g.C_ROW, variant, strict=True)
+
+
+# ------------------------------------------------------------------------------------------------
+# The tuned plan table compiled into the library: every entry at its own shape, through the automatic plan (so the
+# lookup is part of what is tested), against the oracle
+# ------------------------------------------------------------------------------------------------
+def _shipped_plan_entries():
+    import os
+    import re
+    inc = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "gemm_amd", "csrc", "neogemm_default_plan.inc")
+    rows = [tuple(int(x) for x in m.groups()) for m in
+            re.finditer(r"^\{(\d+), (\d+), (\d+), (\d+), (\d+), (\d+), (\d+)\},", open(inc).read(), re.M)]
+    return sorted(r for r in rows if r[0] > 0)
+
+
+@pytest.mark.parametrize("entry", _shipped_plan_entries(), ids=lambda e: "{}x{}x{}-b{}c{}-v{}s{}".format(*e))
+def test_shipped_plan_entries_parity(dev, entry):
+    M, N, K, b_layout, c_layout, variant, split_k = entry
+    assert g.plan(M, N, K, b_layout, c_layout) == (variant, split_k)
+    check_big(dev, M, N, K, seed=M + N + K, b_layout=b_layout, c_layout=c_layout, nrows=64)
