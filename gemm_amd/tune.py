@@ -52,7 +52,7 @@ def time_us(fn, warmup=5, iters=30, preheat_ms=0.0):
     return sorted(batch(per) for _ in range(3))[1]
 
 
-def tune_shape(M, N, K, nbuf=1, log=sys.stderr, b_layout=B_KN, c_layout=C_ROW):
+def tune_shape(M, N, K, nbuf=1, log=sys.stderr, b_layout=B_KN, c_layout=C_ROW, dump=None):
     """Returns (model choice, its time, best choice, its time) for A [M,K], B in `b_layout`, C in `c_layout`."""
     gen = torch.Generator().manual_seed(0)
     A = (torch.randn(M, K, generator=gen) / math.sqrt(K)).to(torch.bfloat16).cuda()
@@ -75,9 +75,16 @@ def tune_shape(M, N, K, nbuf=1, log=sys.stderr, b_layout=B_KN, c_layout=C_ROW):
                 break
             try:
                 # a short look first: a candidate a quarter behind the best so far is not worth a preheated measurement
-                if time_us(lambda: call(v, s), warmup=2, iters=6) > 1.25 * t_best:
+                t_quick = time_us(lambda: call(v, s), warmup=2, iters=6)
+                if t_quick > 1.25 * t_best:
+                    if dump is not None:
+                        dump.append({"M": M, "N": N, "K": K, "b_layout": b_layout, "c_layout": c_layout, "variant": v, "split_k": s,
+                                     "us": round(t_quick, 2), "quick": True})
                     continue
                 t = time_us(lambda: call(v, s), preheat_ms=heat)
+                if dump is not None:
+                    dump.append({"M": M, "N": N, "K": K, "b_layout": b_layout, "c_layout": c_layout, "variant": v, "split_k": s,
+                                 "us": round(t, 2), "quick": False})
             except NeoGemmError as e:
                 if e.status != ERR_UNSUPPORTED:
                     raise
@@ -122,6 +129,8 @@ def main():
     ap.add_argument("--cold-weights-mb", type=float, default=0.0,
                     help="rotate as many B buffers as it takes to exceed this many MB (more than the last-level cache: every "
                          "launch then streams its B from HBM, as a layer's weights are in inference); overrides --nbuf")
+    ap.add_argument("--dump", help="also write every candidate's time to this file, one JSON object per line (for fitting the "
+                                   "cost model; a candidate that the short look dropped carries that look's time and quick: true)")
     ap.add_argument("--b-layout", type=int, default=B_KN, choices=(B_KN, B_NK), help="0: B [K,N], 1: B [N,K]")
     ap.add_argument("--c-layout", type=int, default=C_ROW, choices=(C_ROW, C_COL), help="0: row-major C, 1: column-major")
     args = ap.parse_args()
@@ -144,7 +153,12 @@ def main():
         nbuf = args.nbuf
         if args.cold_weights_mb > 0:
             nbuf = max(2, min(32, int(args.cold_weights_mb * 1e6 // (2.0 * N * K)) + 1))
-        model, t_model, best, t_best = tune_shape(M, N, K, nbuf, b_layout=args.b_layout, c_layout=args.c_layout)
+        dump = [] if args.dump else None
+        model, t_model, best, t_best = tune_shape(M, N, K, nbuf, b_layout=args.b_layout, c_layout=args.c_layout, dump=dump)
+        if dump:
+            with open(args.dump, "a") as f:
+                for d in dump:
+                    f.write(json.dumps(d) + "\n")
         if best != model and t_best < t_model * (1.0 - args.margin):
             table.append({"M": M, "N": N, "K": K, "b_layout": args.b_layout, "c_layout": args.c_layout,
                           "variant": best[0], "split_k": best[1]})

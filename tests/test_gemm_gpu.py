@@ -1037,16 +1037,23 @@ def test_skinny_n_runs_the_transposed_problem(dev):
 
 
 # ------------------------------------------------------------------------------------------------
-# The tuned plan table compiled into the library: every entry at its own shape, through the automatic plan (so the
-# lookup is part of what is tested), against the oracle
+# The tuned plan table compiled into the library, through the automatic plan (so the lookup is part of what is tested),
+# against the oracle: every entry whose B has at most 60 M elements at its own shape, and of the larger ones the smallest
+# per (layouts, variant, split-K) combination that the others do not cover
 # ------------------------------------------------------------------------------------------------
 def _shipped_plan_entries():
     import os
     import re
     inc = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "gemm_amd", "csrc", "neogemm_default_plan.inc")
-    rows = [tuple(int(x) for x in m.groups()) for m in
-            re.finditer(r"^\{(\d+), (\d+), (\d+), (\d+), (\d+), (\d+), (\d+)\},", open(inc).read(), re.M)]
-    return sorted(r for r in rows if r[0] > 0)
+    rows = sorted(tuple(int(x) for x in m.groups()) for m in
+                  re.finditer(r"^\{(\d+), (\d+), (\d+), (\d+), (\d+), (\d+), (\d+)\},", open(inc).read(), re.M))
+    rows = [r for r in rows if r[0] > 0]
+    small = [r for r in rows if r[1] * r[2] <= 60e6]
+    covered, extra = {r[3:] for r in small}, {}
+    for r in rows:
+        if r[1] * r[2] > 60e6 and r[3:] not in covered and (r[3:] not in extra or r[1] * r[2] < extra[r[3:]][1] * extra[r[3:]][2]):
+            extra[r[3:]] = r
+    return small + sorted(extra.values())
 
 
 @pytest.mark.parametrize("entry", _shipped_plan_entries(), ids=lambda e: "{}x{}x{}-b{}c{}-v{}s{}".format(*e))
