@@ -1844,9 +1844,20 @@ static void plan_model(int64_t M, int64_t N, int64_t K, bool aligned, int c_layo
       t = (double)ceil_div(ceil_div(cols, w), (int64_t)cus) * ((double)w * K * 2.0 / 26.9e3 + frags * K * 2.0 / 90.0e3);
       if (t < bytes / 5.9e6) t = bytes / 5.9e6;
     } else {
-      const double wgs = (double)ceil_div(cols, 64), full = __builtin_floor(wgs / cus), frac = wgs / cus - full;
-      const double rounds = full + (frac > 0.0 ? 0.7 + 0.3 * frac : 0.0);
-      t = rounds * ((double)K * 128.0 + (double)rows * K * 2.0) / (rows <= 16 ? 51.0e3 : rows <= 32 ? 43.0e3 : 39.0e3);
+      // B [K,N]: strips of 64 columns.  A workgroup streams its strip at the rate its loads in flight allow, however few
+      // workgroups there are (16 rows x 4096 .. 28672 columns x 3584 .. 28672 deep with weights from HBM: 27 to 35 GB/s per
+      // workgroup from 32 strips to 224; 64 rows: 35 to 46), so a partial round takes as long as a full one, and all of
+      // them together no less than the bytes take at 5 TB/s.
+      // (A problem that stays in the caches streams faster and fills partial rounds better: the earlier fit.)
+      if (bytes > 32e6) {
+        const double wg_us =
+            ((double)K * 128.0 + (double)ceil_div(rows, 16) * 16.0 * K * 2.0) / (rows <= 16 ? 33.0e3 : rows <= 32 ? 34.0e3 : 42.0e3);
+        t = (double)ceil_div(ceil_div(cols, 64), (int64_t)cus) * wg_us;
+      } else {
+        const double wgs = (double)ceil_div(cols, 64), full = __builtin_floor(wgs / cus), frac = wgs / cus - full;
+        const double rounds = full + (frac > 0.0 ? 0.7 + 0.3 * frac : 0.0);
+        t = rounds * ((double)K * 128.0 + (double)rows * K * 2.0) / (rows <= 16 ? 51.0e3 : rows <= 32 ? 43.0e3 : 39.0e3);
+      }
       if (t < stream_us) t = stream_us;
     }
     t += 3.0;

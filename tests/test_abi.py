@@ -89,6 +89,13 @@ def test_plan_for_the_benchmark_configs():
                   (128, 8192, 8192), (100, 4096, 4096)):
         assert _abi.plan(*shape, b_layout=_abi.B_NK)[0] not in streaming
     # unaligned problems go to the generic kernel
+    # B [K,N] with fewer strips of 64 columns than CUs and weights too large for the caches: a strip streams no faster for the
+    # chip being half empty, so split-K tiles take these (16 x 7168 x 7168: 29 us against 37 for the skinny kernel), while a
+    # full round of strips stays on the skinny kernel
+    skinny = (_abi.VARIANT_SKINNY16, _abi.VARIANT_SKINNY32, _abi.VARIANT_SKINNY64)
+    for M in (16, 64):
+        assert _abi.plan(M, 7168, 7168)[0] not in skinny and _abi.plan(M, 3072, 8192)[0] not in skinny
+        assert _abi.plan(M, 12288, 4096)[0] in skinny and _abi.plan(M, 16384, 2048)[0] in skinny
     assert _abi.plan(100, 100, 100, aligned=False) == (_abi.VARIANT_GENERIC, 1)
     assert _abi.workspace_bytes(0, 5, 5) == 0 and _abi.workspace_bytes(5, 5, 0) == 0
 
