@@ -1190,7 +1190,30 @@ struct SkinnyArgs {
   int rot;    // nonzero: workgroup b starts b * rot steps into its waves' shares of K and wraps around
   int strip;  // columns of C per workgroup: 64, or with B [N,K] a smaller multiple of 8 that fills the CUs better
   int ra, rb; // gemm_strip_kernel: stages in the ring of A / of B
+  // gemm_strip_kernel with K split over ksplit workgroups per strip (0 or 1: none): runs of stages_per_split 128-deep
+  // stages; the partial sums go to ws as fp32, [ksplit] matrices of the shape C has in memory, for splitk_reduce_kernel
+  int ksplit, stages_per_split;
+  float* ws;
 };
+// One fragment of partial sums to the split-K workspace: `part` is this split's matrix, dense, laid out as C is in
+// memory (row-major M x N, or N x M for a column-major C).
+template <bool CCOL>
+__device__ __forceinline__ void skinny_store_partial(f32x4 sum, int t, int f, const SkinnyArgs& p, int n0, int lane, float* part) {
+  const uint32_t frow = lane & 15, fq = (uint32_t)lane >> 4;
+  const int row = CCOL ? 16 * t + 4 * (int)fq : 16 * t + (int)frow;
+  const int col = CCOL ? n0 + 16 * f + (int)frow : n0 + 16 * f + 4 * (int)fq;
+  const int col_end = n0 + p.strip < p.N ? n0 + p.strip : p.N;
+  if (row >= p.M || col >= col_end) return;
+  const int fast = CCOL ? row : col, fast_end = CCOL ? p.M : col_end, ld = CCOL ? p.M : p.N;
+  float* wp = part + (CCOL ? (size_t)col * p.M + row : (size_t)row * p.N + col);
+  if (fast + 3 < fast_end && (ld & 3) == 0) {
+    *(f32x4*)wp = sum;
+  } else {
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+      if (fast + r < fast_end) wp[r] = sum[r];
+  }
+}
 // One 16x16 fragment of sums (row fragment t, column fragment f of the strip at column n0) scaled and written to C.
 // The lane's four elements are consecutive along `fast` (n for a row-major C, m for a column-major one).
 template <bool CCOL>
@@ -1467,11 +1490,17 @@ __global__ __launch_bounds__(512) void gemm_strip_kernel(SkinnyArgs p) {
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int quarter = wave & 3;  // the quarter of a stage of its operand this wave loads
-  // workgroup -> strip: consecutive workgroup ids land on different XCDs; id % 8 selects a contiguous run of strips
+  // workgroup -> (split of K, strip): consecutive workgroup ids land on different XCDs; id % 8 selects a contiguous run
+  // of the work order, which walks the strips split by split
   const int per = gridDim.x >> 3, rem = gridDim.x & 7, xcd = blockIdx.x & 7;
-  const int strip_id = xcd * per + (xcd < rem ? xcd : rem) + (blockIdx.x >> 3);
+  const int work = xcd * per + (xcd < rem ? xcd : rem) + (blockIdx.x >> 3);
+  const int ksplit = p.ksplit > 1 ? p.ksplit : 1, nstrips = (int)gridDim.x / ksplit;
+  const int kz = work / nstrips, strip_id = work - kz * nstrips;
   const int n0 = strip_id * p.strip;
-  const int nst = (p.K + STAGE_K - 1) / STAGE_K;
+  // this workgroup's stages of K: [st0, st0 + nst) (the host leaves no split empty)
+  const int nst_all = (p.K + STAGE_K - 1) / STAGE_K;
+  const int st0 = ksplit > 1 ? kz * p.stages_per_split : 0;
+  const int nst = ksplit > 1 ? (p.stages_per_split < nst_all - st0 ? p.stages_per_split : nst_all - st0) : nst_all;
   const int RA = p.ra, RB = p.rb;
   const uint32_t ring_a = lds0, ring_b = lds0 + (uint32_t)RA * A_STAGE;
   const int rot0 = p.rot ? (int)(((unsigned)strip_id * (unsigned)p.rot) % (unsigned)nst) : 0;
@@ -1524,6 +1553,7 @@ __global__ __launch_bounds__(512) void gemm_strip_kernel(SkinnyArgs p) {
       const bool live = s < nst;
       int ps = live ? s + rot0 : 0;
       if (ps >= nst) ps -= nst;
+      ps += st0;
       // depth left from the quarter's first element on (K-major: < 64 is the K tail of its image; B [K,N]: < 32)
       const int krem = live ? p.K - (ps * STAGE_K + kq) : 64;
       const uint64_t b = base0 + (uint64_t)ps * kadv - VOFF_BIAS;
@@ -1621,7 +1651,10 @@ __global__ __launch_bounds__(512) void gemm_strip_kernel(SkinnyArgs p) {
   for (int i = 0; i < RWF; ++i)
 #pragma unroll
     for (int f = 0; f < NF; ++f)
-      if (i < nrf) skinny_store_frag<CCOL>(acc[i][f], rf0 + i, f, p, n0, lane);
+      if (i < nrf) {
+        if (ksplit > 1) skinny_store_partial<CCOL>(acc[i][f], rf0 + i, f, p, n0, lane, p.ws + (size_t)kz * p.M * p.N);
+        else skinny_store_frag<CCOL>(acc[i][f], rf0 + i, f, p, n0, lane);
+      }
 }
 
 // Sum the split-K partials in split order (deterministic) and round once to bf16.
@@ -1829,6 +1862,11 @@ static void plan_model(int64_t M, int64_t N, int64_t K, bool aligned, int c_layo
   // (M <= 16), 96 KiB (M <= 32) or 64 KiB (M <= 64) of B in flight each at ~2.5 us per round trip; no split-K,
   // one launch
   // With B [N,K] and N <= 64 < M the same kernel runs the transposed problem (the wide operand is A then).
+  // Both operands K-major with rows a multiple of 16 KiB apart: the tiles of all workgroups walk along K in step and crowd
+  // onto a few memory channels (128 x 8192 x 8192 streams at 3.6 TB/s where 128 x 4096 x 14336 reaches 4.4), which the
+  // estimates above do not know; the strip kernels start every strip at another depth for this reason.  So against them
+  // the tiles' estimate counts for a fifth more there.
+  const double best_tile = best * (b_layout == NEOGEMM_B_NK && K % 8192 == 0 && bytes > 32e6 ? 1.2 : 1.0);
   const bool skinny_m = M <= 64, skinny_n = !skinny_m && N <= 64 && b_layout == NEOGEMM_B_NK;
   if ((skinny_m || skinny_n) && batch == 1 && K >= 4 * KTILE) {
     const int64_t rows = skinny_m ? M : N, cols = skinny_m ? N : M;  // the kernel's own terms, whatever the layout of C
@@ -1862,7 +1900,7 @@ static void plan_model(int64_t M, int64_t N, int64_t K, bool aligned, int c_layo
     }
     t += 3.0;
     // (the tile estimates come out a little low for shapes that stream from HBM with few rows, see below)
-    if (t < best * (b_layout == NEOGEMM_B_NK && bytes > 32e6 ? 1.04 : 1.0)) {
+    if (t < best_tile * (b_layout == NEOGEMM_B_NK && bytes > 32e6 ? 1.04 : 1.0)) {
       best = t;
       bv = rows <= 16 ? NEOGEMM_VARIANT_SKINNY16 : rows <= 32 ? NEOGEMM_VARIANT_SKINNY32 : NEOGEMM_VARIANT_SKINNY64;
       bs = 1;
@@ -1895,10 +1933,46 @@ static void plan_model(int64_t M, int64_t N, int64_t K, bool aligned, int c_layo
     if (t < stream_us) t = stream_us;
     // (with more than one round of strips the tile estimates are about right: 128 x 28672 x 4096 55 us for the tiles,
     // 59.5 for the strips)
-    if (t < best * (strip_kernel && wgs > cus ? 1.0 : 1.12)) {
+    // (in more than one round of strips the tiles keep their plain estimate: 128 x 28672 x 8192 105 us against 114)
+    if (t < (wgs > cus ? best : best_tile) * (strip_kernel && wgs > cus ? 1.0 : 1.12)) {
       best = t;
       bv = strip_kernel ? NEOGEMM_VARIANT_STRIP : NEOGEMM_VARIANT_SKINNY128;
       bs = 1;
+    }
+    // The strip kernel with K split over s workgroups per strip, for few strips and deep K (128 x 8192 x 8192: 128 strips,
+    // two splits, 38.0 us against 44.0 for split-K tiles; 112 x 4096 x 16384: four, 37 against 47): the same estimate with
+    // a workgroup's bytes divided by s, plus the reduction as for the tiles; 1024 to 8192 deep per split (deeper, tiles
+    // with more splits win: 112 x 8192 x 28672 104 us against 111) and one round of workgroups (in two rounds, and below 97
+    // rows, the measured times are up to half above this estimate).  Against the tiles' estimate it gets the same eighth
+    // as the unsplit strips (112 x 4096 x 11008: 27.9 us against 33.5 for the tiles, 5120 x 5120: 21.6 against 25.9).
+    if (strip_kernel) {
+      const double against_tiles = best_tile > best * 1.12 ? best_tile : best * 1.12;
+      const double limit = bv == NEOGEMM_VARIANT_STRIP ? best : against_tiles;  // the unsplit strips' estimate if they were taken
+      double split_best = 1e300;
+      int split_at = 1;
+      for (int sp : {2, 3, 4, 6, 8}) {
+        if (K / sp < 1024 || (double)ceil_div(cols, 64) * sp > cus) break;
+        if (K / sp > 8192) continue;
+        const int rounds_i = ceil_div((int64_t)ceil_div(cols, 64) * sp, (int64_t)cus);
+        int ws = 64;  // strip width: see launch_strip
+        const int ww = 8 * ceil_div(cols * sp, 8 * (int64_t)rounds_i * (int64_t)cus);
+        if (ww >= 40 && ww < 64) ws = ww;
+        const double wgs_s = (double)ceil_div(cols, ws) * sp, full_s = __builtin_floor(wgs_s / cus), frac_s = wgs_s / cus - full_s;
+        const double rounds_s = full_s + (frac_s > 0.0 ? 0.7 + 0.3 * frac_s : 0.0);
+        const double bytes_s = ((double)K * 2.0 * ws + (double)ceil_div(rows, 16) * 16.0 * K * 2.0) / sp;
+        double ts = 4.7 + rounds_s * bytes_s / 58.0e3;
+        if (ts < stream_us) ts = stream_us;
+        ts += 4.0 + (4.0 * sp + 2.0) * (double)rows * (double)cols / 5.0e6;
+        if (ts < split_best) {
+          split_best = ts;
+          split_at = sp;
+        }
+      }
+      if (split_best < limit) {
+        best = split_best;
+        bv = NEOGEMM_VARIANT_STRIP;
+        bs = split_at;
+      }
     }
   }
   // the 256x256 tile unsplit, K in whole periods of 128, rows from a K-major operand: the kernel that accumulates twice
@@ -2029,7 +2103,10 @@ static int max_planned_split(int64_t M, int64_t N, int64_t K, int64_t batch) {
 }
 
 // Launch of gemm_strip_kernel (65 to 128 rows).  `rings` = 16 * RA + RB forces the ring depths (0: the defaults below).
-static int launch_strip(SkinnyArgs sa, bool bkm, bool ccol, int rings, hipStream_t st) {
+// split_k > 1: that many workgroups per strip, each with a run of 128-deep stages; `ws` takes the partial sums and the
+// reduction kernel follows.
+static int launch_strip(SkinnyArgs sa, bool bkm, bool ccol, int rings, hipStream_t st, int split_k = 1, void* ws = nullptr,
+                        size_t ws_bytes = 0) {
   int cus = 0;
   if (hipError_t e = current_device_cus(&cus); e != hipSuccess) {
     fprintf(stderr, "neogemm: device query failed: %s\n", hipGetErrorString(e));
@@ -2038,9 +2115,24 @@ static int launch_strip(SkinnyArgs sa, bool bkm, bool ccol, int rings, hipStream
   // Strips of 64 columns; of a K-major B (a strip is a set of whole rows then) the multiple of 8 from 40 up that fills
   // the CUs in whole rounds (N = 14336: 256 strips of 56).  Strips of B [K,N] that are not 64 wide would share the cache
   // lines at their edges with their neighbours: 128 x 14336 x 4096 takes 47 us with strips of 56 against 38 with 64.
+  // split K: no empty split, and a workspace of one fp32 matrix per split
+  const int stages = ceil_div(sa.K, 128);
+  if (split_k > stages) split_k = stages;
+  sa.ksplit = 1;
+  if (split_k > 1) {
+    sa.stages_per_split = ceil_div(stages, split_k);
+    sa.ksplit = ceil_div(stages, sa.stages_per_split);
+  }
+  if (sa.ksplit > 1) {
+    if (!ws || ws_bytes < (size_t)sa.ksplit * (size_t)sa.M * (size_t)sa.N * sizeof(float)) return NEOGEMM_ERR_WORKSPACE;
+    if (((uintptr_t)ws & 15) != 0) return NEOGEMM_ERR_BAD_ARG;
+    sa.ws = (float*)ws;
+  }
   sa.strip = 64;
   if (bkm) {
-    const int rounds = ceil_div(ceil_div(sa.N, 64), cus), w = 8 * ceil_div(sa.N, 8 * (int64_t)rounds * cus);
+    // (with K split, the strips of all splits together make the rounds)
+    const int rounds = ceil_div((int64_t)ceil_div(sa.N, 64) * sa.ksplit, cus);
+    const int w = 8 * ceil_div((int64_t)sa.N * sa.ksplit, 8 * (int64_t)rounds * cus);
     if (w >= 40 && w < 64) sa.strip = w;
     sa.rot = 1;  // every strip starts one stage further into K than the one before it: measured 3 to 5 % at K = 4096
   }
@@ -2062,7 +2154,7 @@ static int launch_strip(SkinnyArgs sa, bool bkm, bool ccol, int rings, hipStream
     return NEOGEMM_ERR_UNSUPPORTED;
   auto go = [&](auto kern) -> hipError_t {
     if (hipError_t e = allow_lds(kern, lds); e != hipSuccess) return e;
-    kern<<<dim3(ceil_div(sa.N, sa.strip)), 512, lds, st>>>(sa);
+    kern<<<dim3(ceil_div(sa.N, sa.strip) * sa.ksplit), 512, lds, st>>>(sa);
     return hipGetLastError();
   };
   auto pick = [&](auto tc) -> hipError_t {
@@ -2080,6 +2172,17 @@ static int launch_strip(SkinnyArgs sa, bool bkm, bool ccol, int rings, hipStream
   if (e != hipSuccess) {
     fprintf(stderr, "neogemm: strip kernel launch failed: %s\n", hipGetErrorString(e));
     return NEOGEMM_ERR_LAUNCH;
+  }
+  if (sa.ksplit > 1) {
+    // C as it lies in memory: M x N row-major, or N x M for a column-major C
+    const int rows_mem = ccol ? sa.N : sa.M, cols_mem = ccol ? sa.M : sa.N;
+    const size_t MN = (size_t)sa.M * sa.N;
+    splitk_reduce_kernel<<<dim3((unsigned)((MN + 1023) / 1024), 1), 256, 0, st>>>(sa.ws, sa.C, rows_mem, cols_mem, sa.ldc, sa.ksplit,
+                                                                                sa.alpha, sa.beta, 0);
+    if (hipError_t e2 = hipGetLastError(); e2 != hipSuccess) {
+      fprintf(stderr, "neogemm: split-K reduction launch failed: %s\n", hipGetErrorString(e2));
+      return NEOGEMM_ERR_LAUNCH;
+    }
   }
   return NEOGEMM_OK;
 }
@@ -2149,7 +2252,8 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
     // C^T = B * A^T: its small operand is B then, its wide one A, and the layout of C flips.
     const bool swap = M > kVariants[v].bm && N <= kVariants[v].bm && b_layout == NEOGEMM_B_NK;
     const bool ok = bt.count == 1 && (M <= kVariants[v].bm || swap) &&
-                    (b_layout == NEOGEMM_B_NK || (N & 7) == 0) && (split_k <= 1 || variant == NEOGEMM_VARIANT_AUTO) && !prof;
+                    (b_layout == NEOGEMM_B_NK || (N & 7) == 0) &&
+                    (split_k <= 1 || variant == NEOGEMM_VARIANT_AUTO || v == NEOGEMM_VARIANT_STRIP) && !prof;
     if (!ok) {
       if (variant != NEOGEMM_VARIANT_AUTO) return NEOGEMM_ERR_UNSUPPORTED;
       // the 128x128 tile needs the least of the tile kernels, then the generic kernel
@@ -2169,7 +2273,7 @@ static int run(const void* A, const void* B, void* C, int64_t M, int64_t N, int6
     }
     const bool wide = v == NEOGEMM_VARIANT_SKINNY128;
     sa.rot = bkm && sa.ldb % 8192 == 0;  // rows of the wide operand a multiple of 16 KiB apart
-    if (v == NEOGEMM_VARIANT_STRIP) return launch_strip(sa, bkm, ccol, group_m, st);
+    if (v == NEOGEMM_VARIANT_STRIP) return launch_strip(sa, bkm, ccol, group_m, st, s, workspace, workspace_bytes);
     if (bkm) {
       // A strip of a K-major B may start at any row of it and be of any width that is a multiple of 8: the width is
       // chosen so that whole rounds of strips fill the CUs (N = 14336: 256 strips of 56 columns instead of 224 of 64,

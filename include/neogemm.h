@@ -74,8 +74,11 @@ extern "C" {
    the skinny variants, but eight waves per workgroup and K in stages of 128 held in rings that the waves share: four
    waves compute (a quarter of the rows each, so no partial sums meet at the end) and request B, four request A and do
    nothing else.  One launch, no workspace; chosen from 97 rows on when the wide operand is K-major and one round of
-   strips about fills the CUs.  For this variant the group_m argument of neogemm_bf16_variant carries the ring depths,
-   16 * stages of A + stages of B (0: the defaults); rings that do not fit the 160 KiB of LDS are refused. */
+   strips about fills the CUs.  With split_k > 1 that many workgroups share a strip, each with a run of 128-deep stages
+   of K, the partial sums go through the workspace (split_k * M * N floats) and the reduction kernel follows: chosen
+   when there are too few strips for the CUs and K is deep (128 x 8192 x 8192: two splits).  For this variant the group_m
+   argument of neogemm_bf16_variant carries the ring depths, 16 * stages of A + stages of B (0: the defaults); rings that
+   do not fit the 160 KiB of LDS are refused. */
 #define NEOGEMM_VARIANT_STRIP 17
 #define NEOGEMM_VARIANT_COUNT 18
 

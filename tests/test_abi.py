@@ -85,9 +85,14 @@ def test_plan_for_the_benchmark_configs():
     assert _abi.plan(128, 14336, 4096, b_layout=_abi.B_KN)[0] not in (_abi.VARIANT_SKINNY128, _abi.VARIANT_STRIP)
     assert _abi.plan(128, 8192, 2048, b_layout=_abi.B_NK) == (_abi.VARIANT_STRIP, 1)   # 14.8 us against 19.1 for split-K tiles
     streaming = (_abi.VARIANT_SKINNY128, _abi.VARIANT_STRIP)
-    for shape in ((128, 28672, 4096), (128, 4096, 14336), (128, 14336, 1024), (96, 6144, 4096), (129, 14336, 4096),
-                  (128, 8192, 8192), (100, 4096, 4096)):
+    for shape in ((128, 28672, 4096), (128, 14336, 1024), (96, 6144, 4096), (129, 14336, 4096), (128, 8192, 28672)):
         assert _abi.plan(*shape, b_layout=_abi.B_NK)[0] not in streaming
+    # few strips and deep K: the strip kernel with K split over the workgroups of a strip, one round of them in all
+    # (128 x 8192 x 8192: 128 strips x 2, 38 us against 44 for split-K tiles), in the transposed problem as well
+    assert _abi.plan(128, 8192, 8192, b_layout=_abi.B_NK) == (_abi.VARIANT_STRIP, 2)
+    assert _abi.plan(112, 4096, 16384, b_layout=_abi.B_NK) == (_abi.VARIANT_STRIP, 4)
+    assert _abi.plan(8192, 128, 8192, b_layout=_abi.B_NK, c_layout=_abi.C_COL) == (_abi.VARIANT_STRIP, 2)
+    assert _abi.workspace_bytes(128, 8192, 8192) >= 2 * 128 * 8192 * 4
     # unaligned problems go to the generic kernel
     # B [K,N] with fewer strips of 64 columns than CUs and weights too large for the caches: a strip streams no faster for the
     # chip being half empty, so split-K tiles take these (16 x 7168 x 7168: 29 us against 37 for the skinny kernel), while a
@@ -217,8 +222,8 @@ def test_shipped_plan_table():
         assert b in (0, 1) and c in (0, 1) and 1 <= s <= 64 and s * 128 <= K
         assert v in tile_variants + (_abi.VARIANT_SKINNY16, _abi.VARIANT_SKINNY32, _abi.VARIANT_SKINNY64, _abi.VARIANT_SKINNY128,
                                      _abi.VARIANT_STRIP)
-        if v in (_abi.VARIANT_C256x256_W4, _abi.VARIANT_STRIP) or v >= _abi.VARIANT_SKINNY16 and v <= _abi.VARIANT_SKINNY64:
-            assert s == 1
+        if v in (_abi.VARIANT_C256x256_W4, _abi.VARIANT_SKINNY128) or v >= _abi.VARIANT_SKINNY16 and v <= _abi.VARIANT_SKINNY64:
+            assert s == 1      # (the strip kernel is the one streaming kernel that splits K)
         assert _abi.plan(M, N, K, b, c) == (v, s), (M, N, K, b, c)
         assert _abi.workspace_bytes(M, N, K) >= (s * M * N * 4 if s > 1 else 0)
         assert _abi.plan(M, N, K, b, c, aligned=False) == (_abi.VARIANT_GENERIC, 1)   # the table is for the MFMA path only

@@ -980,6 +980,45 @@ def test_strip_kernel_known_answers_rings_and_refusals(dev):
     torch.cuda.synchronize()
 
 
+def test_strip_kernel_with_k_split(dev):
+    """The strip kernel with K split over the workgroups of a strip: fp32 partial sums in the workspace, laid out as C is in
+    memory, and the reduction kernel behind it.  Against the oracle on every layout pair, odd shapes and split counts (a split
+    that would be empty is dropped), the transposed problem, twice in a row on one workspace (bit for bit the same); exact on
+    small integers; a workspace that is too small is refused; and the plan sends few strips with deep K there."""
+    lib = _abi.load()
+    for (M, N, K) in ((128, 1024, 1024), (100, 2048, 4096), (120, 520, 2120), (65, 264, 392), (112, 4096, 14336)):
+        for split_k in (2, 3, 8):
+            for b_layout, c_layout in ((g.B_NK, g.C_ROW), (g.B_NK, g.C_COL), (g.B_KN, g.C_ROW), (g.B_KN, g.C_COL)):
+                if c_layout == g.C_COL and M % 4:
+                    continue
+                A, Bkn = o.make_inputs(M, N, K, seed=M + N + K + split_k)
+                got = [run_abi(A, layouts(Bkn, b_layout), dev, b_layout, c_layout, g.VARIANT_STRIP, split_k) for _ in range(2)]
+                assert torch.equal(got[0], got[1])
+                o.assert_parity(got[0], A, Bkn, what=f"strip {M}x{N}x{K} split {split_k} b{b_layout} c{c_layout}")
+    for (M, N, K, split_k) in ((4096, 128, 4096, 2), (8192, 100, 2048, 4)):      # 65 .. 128 columns, B [N,K]: C^T = B * A^T
+        for c_layout in (g.C_ROW, g.C_COL):
+            A, Bkn = o.make_inputs(M, N, K, seed=M + N)
+            got = run_abi(A, Bkn.t().contiguous(), dev, g.B_NK, c_layout, g.VARIANT_STRIP, split_k)
+            o.assert_parity(got, A, Bkn, what=f"strip transposed {M}x{N}x{K} split {split_k} c{c_layout}")
+    gen = torch.Generator().manual_seed(41)
+    M, N, K = 128, 512, 1024
+    A = torch.randint(-3, 4, (M, K), generator=gen).to(torch.bfloat16)
+    B = torch.randint(-3, 4, (K, N), generator=gen).to(torch.bfloat16)
+    for b_layout in (g.B_KN, g.B_NK):
+        got = run_abi(A, layouts(B, b_layout), dev, b_layout, g.C_ROW, g.VARIANT_STRIP, 4)
+        assert np.array_equal(o.bits_of(got), o.bits_of(o.ref_gemm(A, B)))
+    Ad, Bd = A.to(dev), B.to(dev)
+    C = torch.zeros(M, N, dtype=torch.bfloat16, device=dev)
+    ws = torch.zeros(4 * M * N, dtype=torch.float32, device=dev)
+    call = lambda nbytes: lib.neogemm_bf16_variant(Ad.data_ptr(), Bd.data_ptr(), C.data_ptr(), M, N, K, K, N, N, g.B_KN, g.C_ROW,
+                                                   ws.data_ptr(), nbytes, None, g.VARIANT_STRIP, 4, 0)
+    assert call(4 * M * N * 4 - 16) == _abi.ERR_WORKSPACE and call(4 * M * N * 4) == _abi.OK
+    torch.cuda.synchronize()
+    assert g.plan(128, 8192, 8192, b_layout=g.B_NK) == (g.VARIANT_STRIP, 2)
+    check_big(dev, 128, 8192, 8192, seed=5, b_layout=g.B_NK)
+    check_big(dev, 8192, 128, 8192, seed=6, b_layout=g.B_NK, c_layout=g.C_COL)
+
+
 def test_strip_kernel_on_the_transposed_problem_and_through_the_plan(dev):
     """N in 97 .. 128 < M with B [N,K] runs C^T = B * A^T on the strip kernel; the plan sends 97 to 128 rows with a K-major
     wide operand there when one round of strips about fills the CUs."""
