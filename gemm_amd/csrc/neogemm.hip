@@ -1867,6 +1867,33 @@ static void plan_model(int64_t M, int64_t N, int64_t K, bool aligned, int c_layo
   // estimates above do not know; the strip kernels start every strip at another depth for this reason.  So against them
   // the tiles' estimate counts for a fifth more there.
   const double best_tile = best * (b_layout == NEOGEMM_B_NK && K % 8192 == 0 && bytes > 32e6 ? 1.2 : 1.0);
+  // The strip kernel with K split over s workgroups per strip, for few strips and deep K (128 x 8192 x 8192: 128 strips,
+  // two splits, 38.0 us against 44.0 for split-K tiles; 112 x 4096 x 16384: four, 37 against 47): the unsplit kernel's
+  // estimate with a workgroup's bytes divided by s, plus the reduction as for the tiles; 1024 to 8192 deep per split
+  // (deeper, tiles with more splits win: 112 x 8192 x 28672 104 us against 111) and one round of workgroups (in two
+  // rounds the measured times are up to half above this estimate).  Returns the best split and its estimate.
+  auto strip_split = [&](int64_t srows, int64_t scols, int* split_at) {
+    double split_best = 1e300;
+    for (int sp : {2, 3, 4, 6, 8}) {
+      if (K / sp < 1024 || (double)ceil_div(scols, 64) * sp > cus) break;
+      if (K / sp > 8192) continue;
+      const int rounds_i = ceil_div((int64_t)ceil_div(scols, 64) * sp, (int64_t)cus);
+      int ws = 64;  // strip width: see launch_strip
+      const int ww = 8 * ceil_div(scols * sp, 8 * (int64_t)rounds_i * (int64_t)cus);
+      if (ww >= 40 && ww < 64) ws = ww;
+      const double wgs_s = (double)ceil_div(scols, ws) * sp, full_s = __builtin_floor(wgs_s / cus), frac_s = wgs_s / cus - full_s;
+      const double rounds_s = full_s + (frac_s > 0.0 ? 0.7 + 0.3 * frac_s : 0.0);
+      const double bytes_s = ((double)K * 2.0 * ws + (double)ceil_div(srows, 16) * 16.0 * K * 2.0) / sp;
+      double ts = 4.7 + rounds_s * bytes_s / 58.0e3;
+      if (ts < stream_us) ts = stream_us;
+      ts += 4.0 + (4.0 * sp + 2.0) * (double)srows * (double)scols / 5.0e6;
+      if (ts < split_best) {
+        split_best = ts;
+        *split_at = sp;
+      }
+    }
+    return split_best;
+  };
   const bool skinny_m = M <= 64, skinny_n = !skinny_m && N <= 64 && b_layout == NEOGEMM_B_NK;
   if ((skinny_m || skinny_n) && batch == 1 && K >= 4 * KTILE) {
     const int64_t rows = skinny_m ? M : N, cols = skinny_m ? N : M;  // the kernel's own terms, whatever the layout of C
@@ -1900,10 +1927,25 @@ static void plan_model(int64_t M, int64_t N, int64_t K, bool aligned, int c_layo
     }
     t += 3.0;
     // (the tile estimates come out a little low for shapes that stream from HBM with few rows, see below)
+    bool took_skinny = false;
     if (t < best_tile * (b_layout == NEOGEMM_B_NK && bytes > 32e6 ? 1.04 : 1.0)) {
       best = t;
       bv = rows <= 16 ? NEOGEMM_VARIANT_SKINNY16 : rows <= 32 ? NEOGEMM_VARIANT_SKINNY32 : NEOGEMM_VARIANT_SKINNY64;
       bs = 1;
+      took_skinny = true;
+    }
+    // 33 to 64 rows of a K-major wide operand, few strips, deep K: the strip kernel with K split (64 x 4096 x 16384: four
+    // splits, 30.6 us against 38.1 for the tiles; 64 x 8192 x 8192: two, 31.7 against 33.7 for the skinny kernel); with
+    // fewer rows it loses to the skinny kernel (16 x 8192 x 8192: 29.6 against 27.4)
+    if (b_layout == NEOGEMM_B_NK && rows > 32) {
+      int sp = 1;
+      const double ts = strip_split(rows, cols, &sp);
+      const double against_tiles = best_tile > best * 1.12 ? best_tile : best * 1.12;
+      if (ts < (took_skinny ? best : against_tiles)) {
+        best = ts;
+        bv = NEOGEMM_VARIANT_STRIP;
+        bs = sp;
+      }
     }
   }
   // 65 to 128 rows (of M, or of N with B [N,K]): strips again, one launch, no workspace.  Up to 96 rows, and with
@@ -1939,39 +1981,18 @@ static void plan_model(int64_t M, int64_t N, int64_t K, bool aligned, int c_layo
       bv = strip_kernel ? NEOGEMM_VARIANT_STRIP : NEOGEMM_VARIANT_SKINNY128;
       bs = 1;
     }
-    // The strip kernel with K split over s workgroups per strip, for few strips and deep K (128 x 8192 x 8192: 128 strips,
-    // two splits, 38.0 us against 44.0 for split-K tiles; 112 x 4096 x 16384: four, 37 against 47): the same estimate with
-    // a workgroup's bytes divided by s, plus the reduction as for the tiles; 1024 to 8192 deep per split (deeper, tiles
-    // with more splits win: 112 x 8192 x 28672 104 us against 111) and one round of workgroups (in two rounds, and below 97
-    // rows, the measured times are up to half above this estimate).  Against the tiles' estimate it gets the same eighth
-    // as the unsplit strips (112 x 4096 x 11008: 27.9 us against 33.5 for the tiles, 5120 x 5120: 21.6 against 25.9).
+    // K split over the workgroups of a strip (see strip_split above), from 97 rows on here (65 to 96: up to half above
+    // the estimate).  Against the tiles' estimate it gets the same eighth as the unsplit strips (112 x 4096 x 11008: 27.9 us
+    // against 33.5 for the tiles, 5120 x 5120: 21.6 against 25.9).
     if (strip_kernel) {
       const double against_tiles = best_tile > best * 1.12 ? best_tile : best * 1.12;
       const double limit = bv == NEOGEMM_VARIANT_STRIP ? best : against_tiles;  // the unsplit strips' estimate if they were taken
-      double split_best = 1e300;
-      int split_at = 1;
-      for (int sp : {2, 3, 4, 6, 8}) {
-        if (K / sp < 1024 || (double)ceil_div(cols, 64) * sp > cus) break;
-        if (K / sp > 8192) continue;
-        const int rounds_i = ceil_div((int64_t)ceil_div(cols, 64) * sp, (int64_t)cus);
-        int ws = 64;  // strip width: see launch_strip
-        const int ww = 8 * ceil_div(cols * sp, 8 * (int64_t)rounds_i * (int64_t)cus);
-        if (ww >= 40 && ww < 64) ws = ww;
-        const double wgs_s = (double)ceil_div(cols, ws) * sp, full_s = __builtin_floor(wgs_s / cus), frac_s = wgs_s / cus - full_s;
-        const double rounds_s = full_s + (frac_s > 0.0 ? 0.7 + 0.3 * frac_s : 0.0);
-        const double bytes_s = ((double)K * 2.0 * ws + (double)ceil_div(rows, 16) * 16.0 * K * 2.0) / sp;
-        double ts = 4.7 + rounds_s * bytes_s / 58.0e3;
-        if (ts < stream_us) ts = stream_us;
-        ts += 4.0 + (4.0 * sp + 2.0) * (double)rows * (double)cols / 5.0e6;
-        if (ts < split_best) {
-          split_best = ts;
-          split_at = sp;
-        }
-      }
-      if (split_best < limit) {
-        best = split_best;
+      int sp = 1;
+      const double ts = strip_split(rows, cols, &sp);
+      if (ts < limit) {
+        best = ts;
         bv = NEOGEMM_VARIANT_STRIP;
-        bs = split_at;
+        bs = sp;
       }
     }
   }
@@ -2136,11 +2157,14 @@ static int launch_strip(SkinnyArgs sa, bool bkm, bool ccol, int rings, hipStream
     if (w >= 40 && w < 64) sa.strip = w;
     sa.rot = 1;  // every strip starts one stage further into K than the one before it: measured 3 to 5 % at K = 4096
   }
-  const int tmf = ceil_div(sa.M, 16);
-  if (tmf < 5 || tmf > 8) return NEOGEMM_ERR_UNSUPPORTED;
+  // row fragments of 16: five to eight, or four for up to 64 rows when K is split (unsplit, gemm_skinny_kernel is the
+  // kernel for those; rows past M are zero fills that touch no memory)
+  int tmf = ceil_div(sa.M, 16);
+  if (tmf < 4 && sa.ksplit > 1) tmf = 4;
+  if (tmf < (sa.ksplit > 1 ? 4 : 5) || tmf > 8) return NEOGEMM_ERR_UNSUPPORTED;
   // ring depths: three stages of A (4 KiB * tmf each: two in flight cover the way to L2 and back) and what the 160 KiB
   // leave for B (16 KiB a stage)
-  static const int kRings[9][2] = {{0, 0}, {0, 0}, {0, 0}, {0, 0}, {0, 0}, {3, 6}, {3, 5}, {3, 4}, {3, 4}};
+  static const int kRings[9][2] = {{0, 0}, {0, 0}, {0, 0}, {0, 0}, {3, 6}, {3, 6}, {3, 5}, {3, 4}, {3, 4}};
   sa.ra = kRings[tmf][0];
   sa.rb = kRings[tmf][1];
   if (rings > 0) {
@@ -2164,6 +2188,7 @@ static int launch_strip(SkinnyArgs sa, bool bkm, bool ccol, int rings, hipStream
   };
   hipError_t e = hipErrorInvalidValue;
   switch (tmf) {
+    case 4: e = pick(std::integral_constant<int, 4>{}); break;
     case 5: e = pick(std::integral_constant<int, 5>{}); break;
     case 6: e = pick(std::integral_constant<int, 6>{}); break;
     case 7: e = pick(std::integral_constant<int, 7>{}); break;

@@ -88,7 +88,7 @@ def tune_shape(M, N, K, nbuf=1, log=sys.stderr, b_layout=B_KN, c_layout=C_ROW, d
             except NeoGemmError as e:
                 if e.status != ERR_UNSUPPORTED:
                     raise
-                break
+                continue   # (a variant may refuse a shape unsplit and take it split: the strip kernel up to 64 rows)
             if t < t_best:
                 best, t_best = (v, s), t
     t_model = min(t_model, time_us(lambda: call(None, 0), preheat_ms=heat))   # the first measurement ran on a cold clock

@@ -91,6 +91,8 @@ def test_plan_for_the_benchmark_configs():
     # (128 x 8192 x 8192: 128 strips x 2, 38 us against 44 for split-K tiles), in the transposed problem as well
     assert _abi.plan(128, 8192, 8192, b_layout=_abi.B_NK) == (_abi.VARIANT_STRIP, 2)
     assert _abi.plan(112, 4096, 16384, b_layout=_abi.B_NK) == (_abi.VARIANT_STRIP, 4)
+    assert _abi.plan(64, 8192, 8192, b_layout=_abi.B_NK) == (_abi.VARIANT_STRIP, 2)      # 31.7 us against 33.7 for the skinny kernel
+    assert _abi.plan(16, 8192, 8192, b_layout=_abi.B_NK) == (_abi.VARIANT_SKINNY16, 1)   # 27.4 against 29.6
     assert _abi.plan(8192, 128, 8192, b_layout=_abi.B_NK, c_layout=_abi.C_COL) == (_abi.VARIANT_STRIP, 2)
     assert _abi.workspace_bytes(128, 8192, 8192) >= 2 * 128 * 8192 * 4
     # unaligned problems go to the generic kernel

@@ -986,7 +986,9 @@ def test_strip_kernel_with_k_split(dev):
     that would be empty is dropped), the transposed problem, twice in a row on one workspace (bit for bit the same); exact on
     small integers; a workspace that is too small is refused; and the plan sends few strips with deep K there."""
     lib = _abi.load()
-    for (M, N, K) in ((128, 1024, 1024), (100, 2048, 4096), (120, 520, 2120), (65, 264, 392), (112, 4096, 14336)):
+    # (with K split the kernel also takes 64 rows and fewer, on four row fragments: unsplit those are refused)
+    for (M, N, K) in ((128, 1024, 1024), (100, 2048, 4096), (120, 520, 2120), (65, 264, 392), (112, 4096, 14336), (64, 1024, 1024),
+                      (40, 2048, 4096), (16, 520, 2120), (1, 264, 392)):
         for split_k in (2, 3, 8):
             for b_layout, c_layout in ((g.B_NK, g.C_ROW), (g.B_NK, g.C_COL), (g.B_KN, g.C_ROW), (g.B_KN, g.C_COL)):
                 if c_layout == g.C_COL and M % 4:
@@ -1014,7 +1016,11 @@ def test_strip_kernel_with_k_split(dev):
                                                    ws.data_ptr(), nbytes, None, g.VARIANT_STRIP, 4, 0)
     assert call(4 * M * N * 4 - 16) == _abi.ERR_WORKSPACE and call(4 * M * N * 4) == _abi.OK
     torch.cuda.synchronize()
+    with pytest.raises(g.NeoGemmError):
+        run_abi(A[:64], B, dev, g.B_KN, g.C_ROW, g.VARIANT_STRIP, 1)
     assert g.plan(128, 8192, 8192, b_layout=g.B_NK) == (g.VARIANT_STRIP, 2)
+    assert g.plan(64, 8192, 8192, b_layout=g.B_NK) == (g.VARIANT_STRIP, 2) and g.plan(16, 8192, 8192, b_layout=g.B_NK)[0] == g.VARIANT_SKINNY16
+    check_big(dev, 64, 8192, 8192, seed=7, b_layout=g.B_NK)
     check_big(dev, 128, 8192, 8192, seed=5, b_layout=g.B_NK)
     check_big(dev, 8192, 128, 8192, seed=6, b_layout=g.B_NK, c_layout=g.C_COL)
 
