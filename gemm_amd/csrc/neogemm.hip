@@ -1850,6 +1850,15 @@ static void plan_model(int64_t M, int64_t N, int64_t K, bool aligned, int c_layo
       const double fill = wgs < cus ? wgs / cus : 1.0;
       const double floor_us = stream_us / (0.55 + 0.45 * fill);
       if (t < floor_us) t = floor_us;
+      // Few rows against weights that stream from HBM: every further tile along the short side requests the weights again,
+      // from the L2s, which is not free when the launch lives on its loads: 50 ns per MB (512 x 7168 x 7168 with B [N,K]:
+      // four row tiles of 128, 72 us; two of 256, 62).  Fitted to the candidate timings of 16 to 512 rows with cold weights,
+      // where it takes the plan's mean loss against the best candidate from 6.0 % to 3.6 %.
+      if (bytes > 32e6 && (rows <= 512 || cols <= 512)) {
+        const double again = cols >= rows ? (double)(ceil_div(rows, kVariants[c.variant].bm) - 1) * (double)cols
+                                          : (double)(ceil_div(cols, kVariants[c.variant].bn) - 1) * (double)rows;
+        t += again * (double)K * 2.0 * (double)batch * 5.0e-8;
+      }
       if (sp > 1) t += 4.0 + (4.0 * sp + 2.0) * (double)rows * (double)cols * (double)batch / 5.0e6;
       if (t < best) {
         best = t;
