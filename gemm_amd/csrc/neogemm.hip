@@ -1839,9 +1839,11 @@ static void plan_model(int64_t M, int64_t N, int64_t K, bool aligned, int c_layo
       if (c.variant == NEOGEMM_VARIANT_T128x256_W4 && b_layout == NEOGEMM_B_NK) t *= 1.02;
       // latency knows no discount, and two latency-bound workgroups on one CU were measured to take turns
       // (with both operands K-major the 128x128 tile has three tiles of each in flight when it streams: 256 x 14336 x 4096
-      // unsplit, 224 workgroups, runs its 64 K tiles in 32.3 us; with far fewer workgroups than CUs a K tile takes longer)
+      // unsplit, 224 workgroups, runs its 64 K tiles in 32.3 us; with far fewer workgroups than CUs a K tile takes longer,
+      // and with more than CUs the second workgroup of a CU goes at the pace of the first: 128 x 5120 x 27648 with split 6,
+      // 240 workgroups, 69 us; split 8, 320 of them, 98; split 12, 480, 76)
       const double lat_v =
-          c.variant == NEOGEMM_VARIANT_T128x128_W4 && bytes > 32e6 && b_layout == NEOGEMM_B_NK && wgs >= 0.6 * cus ? 0.46 : lat_us;
+          c.variant == NEOGEMM_VARIANT_T128x128_W4 && bytes > 32e6 && b_layout == NEOGEMM_B_NK && wgs >= 0.6 * cus && wgs <= cus ? 0.46 : lat_us;
       const double lat_floor = __builtin_ceil(wgs / cus) * ktps * lat_v;
       if (t < lat_floor) t = lat_floor;
       t += rounds * (c.fixed_us + (sp > 1 ? c.split_fixed_us : 0.0));
@@ -1977,27 +1979,32 @@ static void plan_model(int64_t M, int64_t N, int64_t K, bool aligned, int c_layo
       if (ww >= 40 && ww < 64) w = ww;
     }
     const double wgs = (double)ceil_div(cols, w), full = __builtin_floor(wgs / cus), frac = wgs / cus - full;
-    const double rounds = full + (frac > 0.0 ? 0.7 + 0.3 * frac : 0.0);
+    // (gemm_skinny_kernel with weights from HBM: a partial round of strips takes as long as a full one, 72 x 27648 x 5120
+    // in 432 strips 69 us)
+    const double rounds = !strip_kernel && bytes > 32e6 ? __builtin_ceil(wgs / cus) : full + (frac > 0.0 ? 0.7 + 0.3 * frac : 0.0);
     const double wg_bytes = (double)K * 2.0 * w + (double)ceil_div(rows, 16) * 16.0 * K * 2.0;
     double t = strip_kernel ? 4.7 + rounds * wg_bytes / 58.0e3
                             : 7.0 + rounds * wg_bytes / (b_layout == NEOGEMM_B_NK ? 52.0e3 : 46.0e3);
     if (t < stream_us) t = stream_us;
     // (with more than one round of strips the tile estimates are about right: 128 x 28672 x 4096 55 us for the tiles,
-    // 59.5 for the strips)
+    // 59.5 for the strips; 72 x 27648 x 5120 58 us for the tiles, 69 for gemm_skinny_kernel)
     // (in more than one round of strips the tiles keep their plain estimate: 128 x 28672 x 8192 105 us against 114)
-    if (t < (wgs > cus ? best : best_tile) * (strip_kernel && wgs > cus ? 1.0 : 1.12)) {
+    if (t < (wgs > cus ? best : best_tile) * (wgs > cus ? 1.0 : 1.12)) {
       best = t;
       bv = strip_kernel ? NEOGEMM_VARIANT_STRIP : NEOGEMM_VARIANT_SKINNY128;
       bs = 1;
     }
-    // K split over the workgroups of a strip (see strip_split above), from 97 rows on here (65 to 96: up to half above
-    // the estimate).  Against the tiles' estimate it gets the same eighth as the unsplit strips (112 x 4096 x 11008: 27.9 us
-    // against 33.5 for the tiles, 5120 x 5120: 21.6 against 25.9).
-    if (strip_kernel) {
+    // K split over the workgroups of a strip (see strip_split above).  Against the tiles' estimate it gets the same
+    // eighth as the unsplit strips (112 x 4096 x 11008: 27.9 us against 33.5 for the tiles, 5120 x 5120: 21.6 against
+    // 25.9).  With 65 to 96 rows the time falls less with the rows than the estimate does (72 x 8192 x 8192: 36.6 us,
+    // 128 rows 37.5), so it counts for an eighth more there; it still beats the tiles (72 x 4096 x 16384: 35.8 us
+    // against 44.9).
+    if (b_layout == NEOGEMM_B_NK) {
       const double against_tiles = best_tile > best * 1.12 ? best_tile : best * 1.12;
-      const double limit = bv == NEOGEMM_VARIANT_STRIP ? best : against_tiles;  // the unsplit strips' estimate if they were taken
+      // the unsplit strips' estimate if they were taken
+      const double limit = bv == NEOGEMM_VARIANT_STRIP || bv == NEOGEMM_VARIANT_SKINNY128 ? best : against_tiles;
       int sp = 1;
-      const double ts = strip_split(rows, cols, &sp);
+      const double ts = strip_split(rows, cols, &sp) * (rows > 96 ? 1.0 : 1.12);
       if (ts < limit) {
         best = ts;
         bv = NEOGEMM_VARIANT_STRIP;

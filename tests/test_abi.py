@@ -94,6 +94,16 @@ def test_plan_for_the_benchmark_configs():
     assert _abi.plan(64, 8192, 8192, b_layout=_abi.B_NK) == (_abi.VARIANT_STRIP, 2)      # 31.7 us against 33.7 for the skinny kernel
     assert _abi.plan(16, 8192, 8192, b_layout=_abi.B_NK) == (_abi.VARIANT_SKINNY16, 1)   # 27.4 against 29.6
     assert _abi.plan(8192, 128, 8192, b_layout=_abi.B_NK, c_layout=_abi.C_COL) == (_abi.VARIANT_STRIP, 2)
+    # 65 to 96 rows as well (72 x 8192 x 8192: 36.6 us against 42.9 for the tiles; 80 x 4096 x 16384: 36.2 against 45.1)
+    assert _abi.plan(72, 8192, 8192, b_layout=_abi.B_NK) == (_abi.VARIANT_STRIP, 2)
+    assert _abi.plan(80, 4096, 16384, b_layout=_abi.B_NK) == (_abi.VARIANT_STRIP, 4)
+    assert _abi.plan(8192, 80, 8192, b_layout=_abi.B_NK, c_layout=_abi.C_COL) == (_abi.VARIANT_STRIP, 2)
+    # 128x128 tiles on weights from HBM: a few more workgroups than CUs means a second pass on some CUs at the pace of
+    # the first (128 x 5120 x 27648 with B [N,K]: split 6, 240 workgroups, 69 us; split 8, 320 of them, 98)
+    v, s = _abi.plan(104, 5120, 27648, b_layout=_abi.B_NK)
+    assert not (v == _abi.VARIANT_T128x128_W4 and 256 < 40 * s <= 384)
+    # in several rounds of strips gemm_skinny_kernel loses to the tiles (72 x 27648 x 5120: 69 us against 60)
+    assert _abi.plan(88, 27648, 5120, b_layout=_abi.B_NK)[0] != _abi.VARIANT_SKINNY128
     assert _abi.workspace_bytes(128, 8192, 8192) >= 2 * 128 * 8192 * 4
     # unaligned problems go to the generic kernel
     # B [K,N] with fewer strips of 64 columns than CUs and weights too large for the caches: a strip streams no faster for the
