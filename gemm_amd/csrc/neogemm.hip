@@ -1187,7 +1187,8 @@ struct SkinnyArgs {
   int M, N, K;
   long lda, ldb, ldc;
   float alpha, beta;
-  int rot;    // nonzero: workgroup b starts b * rot steps into its waves' shares of K and wraps around
+  int rot;    // nonzero: workgroup b starts b * rot steps into its waves' shares of K and wraps around (gemm_strip_kernel: at a
+              // stage of its run that is a hash of the strip's number)
   int strip;  // columns of C per workgroup: 64, or with B [N,K] a smaller multiple of 8 that fills the CUs better
   int ra, rb; // gemm_strip_kernel: stages in the ring of A / of B
   // gemm_strip_kernel with K split over ksplit workgroups per strip (0 or 1: none): runs of stages_per_split 128-deep
@@ -1503,7 +1504,8 @@ __global__ __launch_bounds__(512) void gemm_strip_kernel(SkinnyArgs p) {
   const int nst = ksplit > 1 ? (p.stages_per_split < nst_all - st0 ? p.stages_per_split : nst_all - st0) : nst_all;
   const int RA = p.ra, RB = p.rb;
   const uint32_t ring_a = lds0, ring_b = lds0 + (uint32_t)RA * A_STAGE;
-  const int rot0 = p.rot ? (int)(((unsigned)strip_id * (unsigned)p.rot) % (unsigned)nst) : 0;
+  // the stage of its run this workgroup starts at: scattered over the strips (see launch_strip)
+  const int rot0 = p.rot ? (int)((((unsigned)strip_id * 0x9E3779B1u) >> 12) % (unsigned)nst) : 0;
 
   f32x4 acc[RWF][NF];
 #pragma unroll
@@ -2171,7 +2173,12 @@ static int launch_strip(SkinnyArgs sa, bool bkm, bool ccol, int rings, hipStream
     const int rounds = ceil_div((int64_t)ceil_div(sa.N, 64) * sa.ksplit, cus);
     const int w = 8 * ceil_div((int64_t)sa.N * sa.ksplit, 8 * (int64_t)rounds * cus);
     if (w >= 40 && w < 64) sa.strip = w;
-    sa.rot = 1;  // every strip starts one stage further into K than the one before it: measured 3 to 5 % at K = 4096
+    // Every strip starts at another stage of K (and wraps around): measured 3 to 5 % at K = 4096 against all strips at one
+    // depth.  Which stage is a multiplicative hash of the strip's number, not a multiple of it: with one stage (256 bytes)
+    // further per strip the requests of all strips meet on few memory channels where the strips lie 512 KiB apart
+    // (128 x 16384 x 4096: 46.5 us against 34), with two stages at 1 MiB apart (128 x 8192 x 8192 in two splits: 50.5 against
+    // 39), with seven at 448 KiB; the hash measured level with the best multiple at twelve shapes, strips 160 KiB to 2 MiB apart.
+    sa.rot = 1;
   }
   // row fragments of 16: five to eight, or four for up to 64 rows when K is split (unsplit, gemm_skinny_kernel is the
   // kernel for those; rows past M are zero fills that touch no memory)
