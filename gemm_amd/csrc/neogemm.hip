@@ -1187,8 +1187,8 @@ struct SkinnyArgs {
   int M, N, K;
   long lda, ldb, ldc;
   float alpha, beta;
-  int rot;    // nonzero: workgroup b starts b * rot steps into its waves' shares of K and wraps around (gemm_strip_kernel: at a
-              // stage of its run that is a hash of the strip's number)
+  int rot;    // nonzero: workgroup b starts b (b + 1) / 2 steps into its waves' shares of K and wraps around (gemm_strip_kernel:
+              // at a stage of its run that is a hash of the strip's number)
   int strip;  // columns of C per workgroup: 64, or with B [N,K] a smaller multiple of 8 that fills the CUs better
   int ra, rb; // gemm_strip_kernel: stages in the ring of A / of B
   // gemm_strip_kernel with K split over ksplit workgroups per strip (0 or 1: none): runs of stages_per_split 128-deep
@@ -1331,10 +1331,12 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(SkinnyArgs p) {
   // masked (the loads are still issued, as zero fills, so that the count of loads in flight does not depend on K)
   // Rows of a K-major B that lie a multiple of 16 KiB apart (K a multiple of 8192) and are all read at the same depth
   // crowd onto a few memory channels: 16 x 14336 x 8192 runs 20 % faster, K = 16384 44 %, when every workgroup starts
-  // at another depth (other K: -3 .. +2 %, B [K,N]: -1 .. -5 %, so only there).  The order of a wave's sums then
-  // depends on the strip, not on anything that varies from run to run.
+  // at another depth (other K: -3 .. +2 %, B [K,N]: -1 .. -5 %, so only there).  Strip b starts b (b + 1) / 2 steps in,
+  // not b: a fixed number of steps per strip can cancel against the distance between the strips in the address hash of
+  // the memory channels (b steps: 16 x 8192 x 8192, strips 512 KiB apart, 29.1 us; this way 25.8; 14336 and 28672 columns
+  // 1 % slower).  The order of a wave's sums then depends on the strip, not on anything that varies from run to run.
   const int n_mine = s_end > s_begin ? (s_end - s_begin + s_stride - 1) / s_stride : 0;
-  const int rot0 = p.rot && n_mine > 0 ? (int)(strip_id * p.rot) % n_mine : 0;
+  const int rot0 = p.rot && n_mine > 0 ? (int)((((unsigned)strip_id * ((unsigned)strip_id + 1u)) >> 1) % (unsigned)n_mine) : 0;
   auto turn = [&](int s) {  // the step taken at the place of step s
     if (!p.rot || s >= s_end) return s;
     int i = (s - s_begin) / s_stride + rot0;
