@@ -76,8 +76,8 @@ extern "C" {
    nothing else.  One launch, no workspace; chosen from 97 rows on when the wide operand is K-major and one round of
    strips about fills the CUs.  With split_k > 1 that many workgroups share a strip, each with a run of 128-deep stages
    of K, the partial sums go through the workspace (split_k * M * N floats) and the reduction kernel follows: chosen
-   when there are too few strips for the CUs and K is deep (128 x 8192 x 8192: two splits); split, the variant also takes
-   fewer than 65 rows (chosen from 33 on).  For this variant the group_m
+   when there are too few strips for the CUs and K is deep (128 x 8192 x 8192: two splits), from 33 rows on: split, the
+   variant also takes fewer than 65 rows.  For this variant the group_m
    argument of neogemm_bf16_variant carries the ring depths, 16 * stages of A + stages of B (0: the defaults); rings that
    do not fit the 160 KiB of LDS are refused. */
 #define NEOGEMM_VARIANT_STRIP 17
