@@ -2004,7 +2004,11 @@ static void plan_model(int64_t M, int64_t N, int64_t K, bool aligned, int c_layo
     // 128 rows 37.5), so it counts for an eighth more there; it still beats the tiles (72 x 4096 x 16384: 35.8 us
     // against 44.9).
     if (b_layout == NEOGEMM_B_NK) {
-      const double against_tiles = best_tile > best * 1.12 ? best_tile : best * 1.12;
+      // (problems under 80 MB, from 97 rows on: the tiles' estimates with split K come out lower still, 120 x 5120 x 5120 26.5 us
+      // measured for 128x128 with split 6 against 22.0 for the strips with split 3, 104 x 6144 x 4096 23.6 against 20.8; with
+      // 96 rows the two are level, 6144 x 4096 22.8 against 23.7)
+      const double low = bytes < 80e6 && rows > 96 ? 1.3 : 1.12;
+      const double against_tiles = best_tile > best * low ? best_tile : best * low;
       // the unsplit strips' estimate if they were taken
       const double limit = bv == NEOGEMM_VARIANT_STRIP || bv == NEOGEMM_VARIANT_SKINNY128 ? best : against_tiles;
       int sp = 1;

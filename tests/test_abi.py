@@ -87,6 +87,9 @@ def test_plan_for_the_benchmark_configs():
     streaming = (_abi.VARIANT_SKINNY128, _abi.VARIANT_STRIP)
     for shape in ((128, 28672, 4096), (128, 14336, 1024), (96, 6144, 4096), (129, 14336, 4096), (128, 8192, 28672)):
         assert _abi.plan(*shape, b_layout=_abi.B_NK)[0] not in streaming
+    # too few strips for one launch without a split, from 97 rows on: the strips split K (104 x 6144 x 4096: 20.8 us against
+    # 23.6 for the tiles; with 96 rows they are level)
+    assert _abi.plan(100, 6144, 4096, b_layout=_abi.B_NK) == (_abi.VARIANT_STRIP, 2)
     # few strips and deep K: the strip kernel with K split over the workgroups of a strip, one round of them in all
     # (128 x 8192 x 8192: 128 strips x 2, 38 us against 44 for split-K tiles), in the transposed problem as well
     assert _abi.plan(128, 8192, 8192, b_layout=_abi.B_NK) == (_abi.VARIANT_STRIP, 2)
