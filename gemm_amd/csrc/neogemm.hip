@@ -1953,10 +1953,12 @@ static void plan_model(int64_t M, int64_t N, int64_t K, bool aligned, int c_layo
     }
     // 33 to 64 rows of a K-major wide operand, few strips, deep K: the strip kernel with K split (64 x 4096 x 16384: four
     // splits, 30.6 us against 38.1 for the tiles; 64 x 8192 x 8192: two, 31.7 against 33.7 for the skinny kernel); with
-    // fewer rows it loses to the skinny kernel (16 x 8192 x 8192: 29.6 against 27.4)
-    if (b_layout == NEOGEMM_B_NK && rows > 32) {
+    // fewer rows it loses to the skinny kernel (16 x 8192 x 8192: 29.6 against 27.4) but not to the tiles where the
+    // skinny kernel is out (24 x 4096 x 11008: 24.1 us against 28.5).  With B [K,N] from 33 rows on, against the tiles
+    // (56 x 4096 x 11008: 26.1 us against 29.3, 64 x 4096 x 12288: 27.8 against 29.4; 16 x 4096 x 12288: 37 against 27).
+    if ((b_layout == NEOGEMM_B_NK && (rows > 32 || !took_skinny)) || (b_layout == NEOGEMM_B_KN && skinny_m && rows > 32 && !took_skinny)) {
       int sp = 1;
-      const double ts = strip_split(rows, cols, &sp);
+      const double ts = strip_split(rows, cols, &sp) * (b_layout == NEOGEMM_B_KN ? 1.08 : 1.0);
       const double against_tiles = best_tile > best * 1.12 ? best_tile : best * 1.12;
       if (ts < (took_skinny ? best : against_tiles)) {
         best = ts;

@@ -97,6 +97,11 @@ def test_plan_for_the_benchmark_configs():
     assert _abi.plan(64, 8192, 8192, b_layout=_abi.B_NK) == (_abi.VARIANT_STRIP, 2)      # 31.7 us against 33.7 for the skinny kernel
     assert _abi.plan(16, 8192, 8192, b_layout=_abi.B_NK) == (_abi.VARIANT_SKINNY16, 1)   # 25.8 against 29.6
     assert _abi.plan(8192, 128, 8192, b_layout=_abi.B_NK, c_layout=_abi.C_COL) == (_abi.VARIANT_STRIP, 2)
+    # below 33 rows where the skinny kernel is out (24 x 4096 x 11008: 24.1 us against 28.5 for the tiles), and with B [K,N]
+    # from 33 rows on (64 x 4096 x 12288: 27.8 us against 29.4) but not below (16 x 4096 x 12288: 37 against 27)
+    assert _abi.plan(24, 4096, 12288, b_layout=_abi.B_NK) == (_abi.VARIANT_STRIP, 4)
+    assert _abi.plan(64, 4096, 12288, b_layout=_abi.B_KN) == (_abi.VARIANT_STRIP, 4)
+    assert _abi.plan(16, 4096, 12288, b_layout=_abi.B_KN)[0] != _abi.VARIANT_STRIP
     # 65 to 96 rows as well (72 x 8192 x 8192: 36.6 us against 42.9 for the tiles; 80 x 4096 x 16384: 36.2 against 45.1)
     assert _abi.plan(72, 8192, 8192, b_layout=_abi.B_NK) == (_abi.VARIANT_STRIP, 2)
     assert _abi.plan(80, 4096, 16384, b_layout=_abi.B_NK) == (_abi.VARIANT_STRIP, 4)
